@@ -1,0 +1,288 @@
+// C ABI: argument validation, kernel-path / tile selection and launch.  See include/apnn_tc.h.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "../../include/apnn_tc.h"
+#include "dispatch.h"
+
+namespace {
+
+using apnn::KParams;
+
+int check_dev_ptr(const void *p) {
+  if (p == nullptr) return APNN_ENULL;
+  if ((reinterpret_cast<uintptr_t>(p) & 15u) != 0) return APNN_EALIGN;
+  return APNN_OK;
+}
+
+std::atomic<int> g_cus{-1};
+
+int device_cus() {
+  int c = g_cus.load(std::memory_order_relaxed);
+  if (c >= 0) return c;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    n = 0;
+  }
+  g_cus.store(n, std::memory_order_relaxed);
+  return n;
+}
+
+uint32_t magic_of(int d) { return d >= 2 ? (uint32_t)(((1ull << 32) + (uint32_t)d - 1) / (uint32_t)d) : 0u; }
+
+// largest tile that still gives every compute unit a work-group, else the smallest one
+int choose_tile(int rowsA, int rowsB, bool packed) {
+  static const int ta[apnn::TILE_COUNT] = {64, 32, 16, 16};
+  static const int tb[apnn::TILE_COUNT] = {64, 32, 32, 16};
+  const int last = packed ? apnn::TILE_16x32 : apnn::TILE_16x16;
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;
+  for (int t = 0; t <= last; ++t) {
+    const long long n = (long long)((rowsA + ta[t] - 1) / ta[t]) * ((rowsB + tb[t] - 1) / tb[t]);
+    if (n >= cus) return t;
+  }
+  return last;
+}
+
+int pick_valu_tile(int tile_pin, const KParams &p, bool packed, int *tile) {
+  if (tile_pin == 0) {
+    *tile = choose_tile(p.rowsA, p.rowsB, packed);
+    return APNN_OK;
+  }
+  const int t = tile_pin - 1;
+  if (t >= apnn::TILE_COUNT || (packed && t == apnn::TILE_16x16)) return APNN_EINVAL;
+  *tile = t;
+  return APNN_OK;
+}
+
+int check_epilogue(const apnn_epilogue &e, int rowsB, bool is_conv, int Ho, int Wo) {
+  if (e.mode != APNN_EPI_INT32 && e.mode != APNN_EPI_LOWBITS && e.mode != APNN_EPI_BN) return APNN_EINVAL;
+  if (e.pool != APNN_POOL_NONE && e.pool != APNN_POOL_AVG2X2 && e.pool != APNN_POOL_MAX2X2) return APNN_EINVAL;
+  if (e.mode == APNN_EPI_INT32) {
+    if (e.pool != APNN_POOL_NONE || e.residual != nullptr || e.save_acc != nullptr) return APNN_EINVAL;
+    return APNN_OK;
+  }
+  if (e.out_bits < 1 || e.out_bits > 8) return APNN_EINVAL;
+  if (rowsB % 32 != 0) return APNN_EINVAL;
+  if (e.mode == APNN_EPI_BN && e.thresholds == nullptr) return APNN_ENULL;
+  if (e.pool != APNN_POOL_NONE) {
+    if (!is_conv || (Ho & 1) || (Wo & 1)) return APNN_EINVAL;
+    if (e.residual != nullptr || e.save_acc != nullptr) return APNN_EINVAL;
+  }
+  return APNN_OK;
+}
+
+void fill_epilogue(KParams &p, const apnn_epilogue &e, void *out, long long out_rows) {
+  p.epi = e.mode;
+  p.out_bits = e.out_bits;
+  p.pool = e.pool;
+  p.thr = e.thresholds;
+  p.flip = e.flip;
+  p.resid = e.residual;
+  p.save_acc = e.save_acc;
+  p.out = out;
+  p.out_plane = out_rows * (p.rowsB / 32);
+}
+
+typedef hipError_t (*valu_fn)(int, int, const KParams &, hipStream_t);
+
+valu_fn valu_gemm_fn(int wb, int xb) {
+  if (wb == 1 && xb == 2) return apnn::valu_gemm_1_2_x;
+  if (wb == 1 && xb == 3) return apnn::valu_gemm_1_3_x;
+  if (wb == 1 && xb == 4) return apnn::valu_gemm_1_4_x;
+  if (wb == 2 && xb == 2) return apnn::valu_gemm_2_2_x;
+  return nullptr;
+}
+
+valu_fn valu_conv_fn(int xb, int wb) {
+  if (xb == 2 && wb == 1) return apnn::valu_conv_2_1_x;
+  if (xb == 3 && wb == 1) return apnn::valu_conv_3_1_x;
+  if (xb == 4 && wb == 1) return apnn::valu_conv_4_1_x;
+  if (xb == 2 && wb == 2) return apnn::valu_conv_2_2_x;
+  return nullptr;
+}
+
+int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
+  if (d == nullptr) return APNN_ENULL;
+  int rc;
+  if ((rc = check_dev_ptr(d->W)) || (rc = check_dev_ptr(d->X)) || (rc = check_dev_ptr(d->D))) return rc;
+  if (d->M <= 0 || d->N <= 0 || d->K <= 0 || (d->K % 128) != 0) return APNN_EINVAL;
+  if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
+  if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
+  const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
+  if ((d->path >> 16) != 0 || (path != APNN_PATH_AUTO && path != APNN_PATH_VALU && path != APNN_PATH_MFMA))
+    return APNN_EINVAL;
+  if ((rc = check_epilogue(d->epi, d->N, false, 0, 0))) return rc;
+
+  KParams p{};
+  p.A = static_cast<const uint32_t *>(d->W);
+  p.B = static_cast<const uint32_t *>(d->X);
+  p.rowsA = d->M;
+  p.rowsB = d->N;
+  p.KW = d->K / 32;
+  p.planeA = (long long)d->M * p.KW;
+  p.planeB = (long long)d->N * p.KW;
+  p.sym = d->weight_mode == APNN_WEIGHT_SYMMETRIC;
+  p.wmax = (1 << d->wb) - 1;
+  fill_epilogue(p, d->epi, d->D, d->M);
+
+  if (path == APNN_PATH_MFMA) return APNN_EUNSUPPORTED;
+  valu_fn fn = valu_gemm_fn(d->wb, d->xb);
+  if (fn == nullptr) return APNN_EUNSUPPORTED;
+  int tile;
+  if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
+  return (int)fn(4, tile, p, stream);
+}
+
+int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
+  if (d == nullptr) return APNN_ENULL;
+  int rc;
+  if ((rc = check_dev_ptr(d->W)) || (rc = check_dev_ptr(d->X)) || (rc = check_dev_ptr(d->O))) return rc;
+  if (d->batch <= 0 || d->H <= 0 || d->Wd <= 0 || d->COUT <= 0) return APNN_EINVAL;
+  if (d->cin_pad <= 0 || (d->cin_pad % 32) != 0) return APNN_EINVAL;
+  if (d->R <= 0 || d->S <= 0 || d->stride <= 0 || d->pad < 0) return APNN_EINVAL;
+  if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
+  if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
+  const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
+  if ((d->path >> 16) != 0 || (path != APNN_PATH_AUTO && path != APNN_PATH_VALU && path != APNN_PATH_MFMA))
+    return APNN_EINVAL;
+  if (d->H + 2 * d->pad < d->R || d->Wd + 2 * d->pad < d->S) return APNN_EINVAL;
+  const int Ho = (d->H + 2 * d->pad - d->R) / d->stride + 1;
+  const int Wo = (d->Wd + 2 * d->pad - d->S) / d->stride + 1;
+  if ((rc = check_epilogue(d->epi, d->COUT, true, Ho, Wo))) return rc;
+  const long long pixels = (long long)d->batch * Ho * Wo;
+  const int C32 = d->cin_pad / 32;
+  const long long KW = (long long)d->R * d->S * C32;
+  if (pixels > 0x7fffffffLL || KW > (1 << 20)) return APNN_EINVAL;
+  // a chunk of 4 words must not straddle two taps when 128-bit loads are used
+  const int vw = (C32 % 4 == 0) ? 4 : (C32 % 2 == 0) ? 2 : 1;
+
+  KParams p{};
+  p.A = static_cast<const uint32_t *>(d->X);
+  p.B = static_cast<const uint32_t *>(d->W);
+  p.rowsA = (int)pixels;
+  p.rowsB = d->COUT;
+  p.KW = (int)KW;
+  p.Hs = d->H + (d->halo ? 2 * d->pad : 0);
+  p.Ws = d->Wd + (d->halo ? 2 * d->pad : 0);
+  p.planeA = (long long)d->batch * p.Hs * p.Ws * C32;
+  p.planeB = (long long)d->COUT * KW;
+  p.C32 = C32;
+  p.Ho = Ho;
+  p.Wo = Wo;
+  p.S = d->S;
+  p.stride = d->stride;
+  p.pad = d->halo ? 0 : d->pad;
+  p.magicC32 = magic_of(C32);
+  p.magicS = magic_of(d->S);
+  p.pool_order = d->epi.pool != APNN_POOL_NONE;
+  p.sym = d->weight_mode == APNN_WEIGHT_SYMMETRIC;
+  p.wmax = (1 << d->wb) - 1;
+  fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
+
+  if (path == APNN_PATH_MFMA) return APNN_EUNSUPPORTED;
+  valu_fn fn = valu_conv_fn(d->xb, d->wb);
+  if (fn == nullptr) return APNN_EUNSUPPORTED;
+  int tile;
+  if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
+  return (int)fn(vw, tile, p, stream);
+}
+
+int named_gemm(int want_wb, int want_xb, int mode, const void *W, const void *X, int *D, int M, int N, int K,
+               int wb, int xb, apnn_stream_t s) {
+  if (wb != want_wb || xb != want_xb) return APNN_EINVAL;
+  apnn_gemm_desc d{};
+  d.W = W;
+  d.X = X;
+  d.D = D;
+  d.M = M;
+  d.N = N;
+  d.K = K;
+  d.wb = wb;
+  d.xb = xb;
+  d.weight_mode = APNN_WEIGHT_UNSIGNED;
+  d.epi.mode = mode;
+  d.epi.out_bits = xb;  // the reference decomposes into as many planes as the activations have
+  d.path = APNN_PATH_AUTO;
+  return run_gemm(&d, static_cast<hipStream_t>(s));
+}
+
+int named_conv(int wb, int xb, int mode, int pool, const void *W, const void *X, int *O, int H, int Wd, int CIN,
+               int COUT, apnn_stream_t s) {
+  if (CIN <= 0 || (CIN % 128) != 0) return APNN_EINVAL;
+  apnn_conv_desc d{};
+  d.W = W;
+  d.X = X;
+  d.O = O;
+  d.batch = 1;
+  d.H = H;
+  d.Wd = Wd;
+  d.cin_pad = CIN;
+  d.COUT = COUT;
+  d.R = 3;
+  d.S = 3;
+  d.stride = 1;
+  d.pad = 1;
+  d.halo = 1;
+  d.wb = wb;
+  d.xb = xb;
+  d.weight_mode = APNN_WEIGHT_UNSIGNED;
+  d.epi.mode = mode;
+  d.epi.out_bits = xb;
+  d.epi.pool = pool;
+  d.path = APNN_PATH_AUTO;
+  return run_conv(&d, static_cast<hipStream_t>(s));
+}
+
+}  // namespace
+
+extern "C" {
+
+#define APNN_DEF_GEMM(name, w, a, mode)                                                                       \
+  int name(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s) {      \
+    return named_gemm(w, a, mode, W, X, D, M, N, K, wb, xb, s);                                                \
+  }
+APNN_DEF_GEMM(apmm_w1a2, 1, 2, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w1a3, 1, 3, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w1a4, 1, 4, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w2a2, 2, 2, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w1a2_decompose, 1, 2, APNN_EPI_LOWBITS)
+APNN_DEF_GEMM(apmm_w1a3_decompose, 1, 3, APNN_EPI_LOWBITS)
+APNN_DEF_GEMM(apmm_w1a4_decompose, 1, 4, APNN_EPI_LOWBITS)
+APNN_DEF_GEMM(apmm_w2a2_decompose, 2, 2, APNN_EPI_LOWBITS)
+#undef APNN_DEF_GEMM
+
+#define APNN_DEF_CONV(name, w, a, mode, pool)                                                                  \
+  int name(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT,               \
+           apnn_stream_t s) {                                                                                  \
+    return named_conv(w, a, mode, pool, W, X, Output, Height, Width, CIN, COUT, s);                           \
+  }
+APNN_DEF_CONV(apconv_w1a2, 1, 2, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w1a3, 1, 3, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w1a4, 1, 4, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w2a2, 2, 2, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w1a2_pack, 1, 2, APNN_EPI_LOWBITS, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w1a3_pack, 1, 3, APNN_EPI_LOWBITS, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w1a4_pack, 1, 4, APNN_EPI_LOWBITS, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w2a2_pack, 2, 2, APNN_EPI_LOWBITS, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w1a2_pack_pool, 1, 2, APNN_EPI_LOWBITS, APNN_POOL_AVG2X2)
+APNN_DEF_CONV(APConv_w2a2_pack_pool, 2, 2, APNN_EPI_LOWBITS, APNN_POOL_AVG2X2)
+#undef APNN_DEF_CONV
+
+int apnn_gemm(const apnn_gemm_desc *d, apnn_stream_t s) { return run_gemm(d, static_cast<hipStream_t>(s)); }
+int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s) { return run_conv(d, static_cast<hipStream_t>(s)); }
+
+int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                   apnn_stream_t s) {
+  if (values == nullptr || planes == nullptr) return APNN_ENULL;
+  if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 32) return APNN_EINVAL;
+  return (int)apnn::launch_pack_bits(values, planes, rows, C, cpad, bits, static_cast<hipStream_t>(s));
+}
+
+int apnn_device_cus(void) { return device_cus(); }
+const char *apnn_version(void) { return "apnn-tc-amd 0.1 (gfx950)"; }
+
+}  // extern "C"

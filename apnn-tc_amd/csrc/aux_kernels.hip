@@ -1,0 +1,42 @@
+// Small helper kernels around the hot path.
+#include <hip/hip_runtime.h>
+
+#include "dispatch.h"
+
+namespace apnn {
+
+// Bit-plane packer with the layout of Bit_compression (APNN-TC-nn/src/kernel.cuh:46-77):
+// one wave handles 64 consecutive channels of one row, a ballot per bit yields two MSB-first words.
+__global__ __launch_bounds__(256) void pack_bits_kernel(const uint32_t *__restrict__ values,
+                                                        uint32_t *__restrict__ planes, int rows, int C,
+                                                        int cpad, int bits) {
+  const int lane = threadIdx.x & 63;
+  const int wave_in_block = threadIdx.x >> 6;
+  const int cw = cpad >> 5;              // words per row
+  const int groups = (cpad + 63) >> 6;   // 64-channel groups per row
+  const long long total = (long long)rows * groups;
+  const long long plane_stride = (long long)rows * cw;
+  for (long long g = (long long)blockIdx.x * 4 + wave_in_block; g < total; g += (long long)gridDim.x * 4) {
+    const int row = (int)(g / groups);
+    const int c = (int)(g % groups) * 64 + lane;
+    const uint32_t v = (c < C) ? values[(long long)row * C + c] : 0u;
+    for (int b = 0; b < bits; ++b) {
+      const unsigned long long mask = __ballot((v >> b) & 1u);
+      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
+      const int wi = c >> 5;
+      if ((lane & 31) == 0 && wi < cw) planes[b * plane_stride + (long long)row * cw + wi] = word;
+    }
+  }
+}
+
+hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                            hipStream_t s) {
+  const long long total = (long long)rows * ((cpad + 63) / 64);
+  long long blocks = (total + 3) / 4;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(pack_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, s, values, planes, rows, C, cpad, bits);
+  return hipGetLastError();
+}
+
+}  // namespace apnn

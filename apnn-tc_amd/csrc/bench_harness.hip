@@ -1,0 +1,74 @@
+// Timing loops for the benchmark driver: the counterpart of the timing section of the reference's
+// benchmark mains (APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:526-549), which
+// launch the kernel NUM_PROFILES times between CUDA events.  Built into libapnn_bench.so, which
+// links libapnn_tc.so and calls it only through the C ABI.
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+
+#include "../../include/apnn_tc.h"
+
+namespace {
+
+template <class F>
+int timed_loop(F &&launch, int warmup, int iters, hipStream_t stream, float *event_ms, double *wall_ms) {
+  hipEvent_t e0, e1;
+  hipError_t err;
+  if ((err = hipEventCreate(&e0)) != hipSuccess) return (int)err;
+  if ((err = hipEventCreate(&e1)) != hipSuccess) return (int)err;
+  int rc = 0;
+  for (int i = 0; i < warmup && rc == 0; ++i) rc = launch();
+  if (rc == 0 && (err = hipStreamSynchronize(stream)) != hipSuccess) rc = (int)err;
+  if (rc == 0) {
+    const auto t0 = std::chrono::steady_clock::now();
+    (void)hipEventRecord(e0, stream);
+    for (int i = 0; i < iters && rc == 0; ++i) rc = launch();
+    (void)hipEventRecord(e1, stream);
+    err = hipStreamSynchronize(stream);
+    const auto t1 = std::chrono::steady_clock::now();
+    if (rc == 0 && err != hipSuccess) rc = (int)err;
+    if (rc == 0) {
+      float ms = 0.f;
+      (void)hipEventElapsedTime(&ms, e0, e1);
+      *event_ms = ms;
+      *wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Runs `iters` back-to-back apnn_gemm launches of the same descriptor on `stream` after `warmup`
+// untimed ones.  event_ms: HIP-event time over the timed launches; wall_ms: host wall clock from
+// first launch to stream idle.
+int apnn_bench_gemm(const apnn_gemm_desc *d, int warmup, int iters, apnn_stream_t s, float *event_ms,
+                    double *wall_ms) {
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  return timed_loop([&]() { return apnn_gemm(d, s); }, warmup, iters, stream, event_ms, wall_ms);
+}
+
+int apnn_bench_conv(const apnn_conv_desc *d, int warmup, int iters, apnn_stream_t s, float *event_ms,
+                    double *wall_ms) {
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  return timed_loop([&]() { return apnn_conv(d, s); }, warmup, iters, stream, event_ms, wall_ms);
+}
+
+__global__ void apnn_bench_empty_kernel() {}
+
+// Launch floor of the machine: the same loop around an empty kernel.
+int apnn_bench_empty(int warmup, int iters, apnn_stream_t s, float *event_ms, double *wall_ms) {
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  return timed_loop(
+      [&]() {
+        hipLaunchKernelGGL(apnn_bench_empty_kernel, dim3(1), dim3(64), 0, stream);
+        return (int)hipGetLastError();
+      },
+      warmup, iters, stream, event_ms, wall_ms);
+}
+
+}  // extern "C"

@@ -1,0 +1,25 @@
+// Host-side declarations of the per-(PA,PB) kernel launchers built from valu_inst.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "kparams.h"
+
+namespace apnn {
+
+#define APNN_DECL_VALU(kind, pa, pb) \
+  hipError_t valu_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);
+APNN_DECL_VALU(gemm, 1, 2)
+APNN_DECL_VALU(gemm, 1, 3)
+APNN_DECL_VALU(gemm, 1, 4)
+APNN_DECL_VALU(gemm, 2, 2)
+APNN_DECL_VALU(conv, 2, 1)
+APNN_DECL_VALU(conv, 3, 1)
+APNN_DECL_VALU(conv, 4, 1)
+APNN_DECL_VALU(conv, 2, 2)
+#undef APNN_DECL_VALU
+
+// aux_kernels.hip
+hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                            hipStream_t s);
+
+}  // namespace apnn

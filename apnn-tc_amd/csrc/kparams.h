@@ -1,0 +1,45 @@
+// Kernel-side problem description shared by the VALU and MFMA kernels and the host dispatcher.
+//
+// Every kernel computes  out[a][b] = sum_{i<PA} sum_{j<PB} 2^(i+j) popc(A_i[a] & B_j[b])  over KW
+// 32-bit words, where A is the slow output index and B the fast (contiguous) one:
+//   GEMM entry points : A = W rows (M),      B = X rows (N)
+//   convolution / FC  : A = output pixels,   B = output channels (implicit im2col on A)
+#pragma once
+#include <stdint.h>
+
+namespace apnn {
+
+enum TileSel { TILE_64x64 = 0, TILE_32x32 = 1, TILE_16x32 = 2, TILE_16x16 = 3, TILE_COUNT = 4 };
+
+struct KParams {
+  const uint32_t *A;
+  const uint32_t *B;
+  int rowsA, rowsB;          // logical output size out[rowsA][rowsB]
+  int KW;                    // reduction length in 32-bit words (GEMM: K/32, conv: R*S*C32)
+  long long planeA, planeB;  // plane strides in words
+
+  // implicit im2col (convolution kernels only); halo-stored inputs are expressed as pad = 0 on the
+  // stored frame
+  int Hs, Ws;                // stored input height / width
+  int C32;                   // words per pixel per plane
+  int Ho, Wo;                // output height / width
+  int S;                     // filter width (filter height = KW / (S*C32))
+  int stride, pad;
+  uint32_t magicC32, magicS; // ceil(2^32/d) for d >= 2 (unused when d == 1)
+  int pool_order;            // 1: row index enumerates 2x2 output windows (4 consecutive rows each)
+
+  int sym;                   // symmetric weights: result = 2*raw - wmax * (activation row sum)
+  int wmax;                  // 2^wb - 1
+
+  int epi;                   // APNN_EPI_*
+  int out_bits;
+  int pool;                  // APNN_POOL_*
+  const int32_t *thr;
+  const uint8_t *flip;
+  const int32_t *resid;
+  int32_t *save_acc;
+  void *out;
+  long long out_plane;       // packed output: plane stride in words
+};
+
+}  // namespace apnn

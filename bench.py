@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""Benchmark driver.
+
+Headline metric (BASELINE.json): w1a2 GEMM effective TOPS at M=64, N=K=1024, weights {-1,+1} stored
+as one bit (w = 2b-1), activations unsigned 2-bit, bit-packed along K, int32 output.  One "step" is
+one launch of that GEMM through the C ABI with all operands resident in HBM.  The timed loop runs in
+C++ (libapnn_bench.so), like the timing section of the reference's benchmark main
+(APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:526-549).
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline     : the GEMM kernel against the HBM roofline (algorithmic bytes / HIP-event time per launch)
+  cpu_baseline : the scalar CPU oracle timed on the host cores on the same inputs
+  extra        : the reference-compatible unsigned result, the launch floor, and the other shapes of
+                 the sweep with their own roofline fractions.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
+BASELINE_TOPS = 18.66          # reference README.md:142 (w1a2, M=64, N=K=1024, sm_86)
+
+
+def gemm_bytes(M, N, K, wb, xb):
+    return (wb * M * K + xb * N * K) // 8 + 4 * M * N
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import gpu_util as G
+    import oracle_lib as O
+
+    A = G.A
+    L = A.lib()
+    benchlib = ctypes.CDLL(os.path.join(os.path.dirname(A.LIB_PATH), "libapnn_bench.so"))
+    benchlib.apnn_bench_gemm.argtypes = [ctypes.POINTER(A.GemmDesc), ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    benchlib.apnn_bench_empty.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                          ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    path = {"auto": A.PATH_AUTO, "valu": A.PATH_VALU, "mfma": A.PATH_MFMA}[args.path]
+
+    def make_inputs(M, N, K, wb, xb):
+        W = O.random_planes(np.random.default_rng(0x5EED0001), wb, M, K // 32)
+        X = O.random_planes(np.random.default_rng(0x5EED0002), xb, N, K // 32)
+        return W, X
+
+    def time_gemm(M, N, K, wb, xb, sym, warmup, iters, verify_rows=None):
+        W, X = make_inputs(M, N, K, wb, xb)
+        dW, dX = G.to_dev(W), G.to_dev(X)
+        out = G.dev_empty_i32(M * N, fill=-7)
+        d = A.GemmDesc(W=dW.data_ptr(), X=dX.data_ptr(), D=out.data_ptr(), M=M, N=N, K=K, wb=wb, xb=xb,
+                       weight_mode=sym, path=path)
+        ev, wall = ctypes.c_float(), ctypes.c_double()
+        torch.cuda.synchronize()
+        A.check(benchlib.apnn_bench_gemm(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
+                                         ctypes.byref(wall)), "apnn_bench_gemm")
+        torch.cuda.synchronize()
+        got = G.to_host(out).reshape(M, N)
+        if verify_rows is None:
+            ok = bool(np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=sym, nthreads=os.cpu_count() or 1)))
+        else:
+            ok = True
+            for m in verify_rows:
+                ref = O.gemm_rows(W, X, M, N, K, wb, xb, m, m + 1, sym_w=sym, nthreads=os.cpu_count() or 1)[0]
+                ok = ok and bool(np.array_equal(got[m], ref))
+        return dict(event_ms=ev.value / iters, wall_ms=wall.value / iters, verified=ok, W=W, X=X)
+
+    # ---- headline -----------------------------------------------------------------------------
+    M, N, K, wb, xb = 64, 1024, 1024, 1, 2
+    ops = 2.0 * M * N * K
+    nbytes = gemm_bytes(M, N, K, wb, xb)
+    r = time_gemm(M, N, K, wb, xb, A.WEIGHT_SYMMETRIC, args.warmup, args.steps)
+    tops = ops / (r["wall_ms"] * 1e-3) / 1e12
+    achieved_gbs = nbytes / (r["event_ms"] * 1e-3) / 1e9
+    result = {
+        "metric": "w1a2 GEMM effective TOPS at M=64,N=K=1024",
+        "value": round(tops, 4),
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": round(tops / BASELINE_TOPS, 4),
+        "dtype": "int32 accumulate over 1-bit x 2-bit planes",
+        "data": "synthetic",
+        "config": {"workload": "apnn_gemm w1a2 M=64 N=1024 K=1024, weights 2b-1 (symmetric), int32 out",
+                   "path": args.path, "verified_bit_exact": r["verified"]},
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 6), "traffic": None,
+                     "algorithmic_bytes": nbytes, "kernel_us": round(r["event_ms"] * 1e3, 4)},
+    }
+
+    extra = {}
+    ev, wall = ctypes.c_float(), ctypes.c_double()
+    benchlib.apnn_bench_empty(args.warmup, args.steps, stream, ctypes.byref(ev), ctypes.byref(wall))
+    extra["empty_kernel_us_per_launch"] = round(wall.value / args.steps * 1e3, 4)
+    ru = time_gemm(M, N, K, wb, xb, A.WEIGHT_UNSIGNED, args.warmup, args.steps)
+    extra["unsigned_reference_arithmetic"] = {"tops": round(ops / (ru["wall_ms"] * 1e-3) / 1e12, 4),
+                                              "us": round(ru["wall_ms"] * 1e3, 4), "verified": ru["verified"]}
+
+    if not args.no_extra:
+        shapes = []
+        for (w_, a_) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
+            for nk in (128, 512, 1024):
+                t = time_gemm(64, nk, nk, w_, a_, A.WEIGHT_UNSIGNED, 20, 200)
+                shapes.append({"shape": "w%da%d M=64 N=K=%d" % (w_, a_, nk),
+                               "us": round(t["wall_ms"] * 1e3, 3),
+                               "tops": round(2.0 * 64 * nk * nk / (t["wall_ms"] * 1e-3) / 1e12, 3),
+                               "verified": t["verified"]})
+            for n in (2048, 4096, 8192):
+                iters = {2048: 20, 4096: 10, 8192: 3}[n]
+                t = time_gemm(n, n, n, w_, a_, A.WEIGHT_UNSIGNED, 2, iters, verify_rows=[0, n // 2 + 1, n - 1])
+                tt = 2.0 * n ** 3 / (t["event_ms"] * 1e-3) / 1e12
+                shapes.append({"shape": "w%da%d M=N=K=%d" % (w_, a_, n), "ms": round(t["event_ms"], 4),
+                               "tops": round(tt, 2), "frac_int8_mfma_peak": round(tt / INT8_MFMA_PEAK_TOPS, 4),
+                               "hbm_gbs": round(gemm_bytes(n, n, n, w_, a_) / (t["event_ms"] * 1e-3) / 1e9, 1),
+                               "verified": t["verified"]})
+        extra["shapes"] = shapes
+    result["extra"] = extra
+
+    # ---- CPU baseline: the scalar oracle on the same inputs, host cores ---------------------------
+    if not args.no_cpu:
+        W, X = r["W"], r["X"]
+        ncores = os.cpu_count() or 1
+        def cpu_time(nthreads, budget_s):
+            n, t0 = 0, time.perf_counter()
+            while True:
+                O.gemm(W, X, M, N, K, wb, xb, sym_w=1, nthreads=nthreads)
+                n += 1
+                el = time.perf_counter() - t0
+                if el > budget_s:
+                    return el / n, n
+        t1, n1 = cpu_time(1, 6.0)
+        tn, nn = cpu_time(ncores, 6.0)
+        result["cpu_baseline"] = {
+            "value": round(ops / tn / 1e12, 5), "unit": "TOPS", "cores": ncores, "kind": "port",
+            "sample": "full headline GEMM (M=64,N=K=1024, +-1 weights), %d runs on %d threads; "
+                      "single thread: %.5f TOPS over %d runs" % (nn, ncores, ops / t1 / 1e12, n1),
+            "single_thread_tops": round(ops / t1 / 1e12, 5),
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,160 @@
+/*
+ * apnn_tc.h -- C ABI of the MI355X (gfx950) arbitrary-precision GEMM / convolution library.
+ *
+ * Every entry point is host-callable, takes caller-owned DEVICE buffers (16-byte aligned, as the
+ * reference's int4 loads require), enqueues work on the given HIP stream (NULL = default stream)
+ * and returns without synchronizing.  Return value: 0 on success, a negative APNN_E* code for a
+ * rejected argument (nothing is launched), or a positive hipError_t from the launch.  Nothing here
+ * aborts, allocates device memory or keeps state between calls.
+ *
+ * Reference paths below are relative to the reference checkout:
+ *   LIB = APNN-TC-lib/bmmaTensorCoreGemm/src,  NN = APNN-TC-nn/src
+ *
+ * Data layout (identical to the reference):
+ *   bit-planes are plane-major, LSB plane first, uint32 words; element k of a row is bit k%32 of
+ *   word k/32 (LIB/71_bmmaTensorCoreGemm.cu:362-369);
+ *   GEMM  W:[wb][M][K/32]  X:[xb][N][K/32]  D:[M][N] int32            (LIB/71:362-373)
+ *   conv  X:[xb][H+2][W+2][CIN/32] (halo stored)  W:[wb][COUT][3][3][CIN/32]  O:[H][W][COUT] int32
+ *                                                                    (LIB/51_bmmaTensorCoreGemm.cu:395-411)
+ *   packed outputs: [out_bits][rows][cols/32], column c at bit 31-c%32 (LIB/66_bmmaTensorCoreGemm.cuh:399-404,
+ *   LIB/67_bmmaTensorCoreGemm.cuh:466-477).
+ */
+#ifndef APNN_TC_H
+#define APNN_TC_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APNN_OK            0
+#define APNN_EINVAL      (-1)  /* dimension / bit-width / mode outside the supported set */
+#define APNN_ENULL       (-2)  /* required pointer is NULL */
+#define APNN_EALIGN      (-3)  /* operand not 16-byte aligned */
+#define APNN_EUNSUPPORTED (-4) /* valid request that no kernel in this build serves */
+
+typedef void *apnn_stream_t; /* a hipStream_t */
+
+/* ---- reference kernel entry points --------------------------------------------------------- */
+
+/* D[m][n] = sum_{i<xb} sum_{j<wb} 2^(i+j) popc(W_j[m] & X_i[n]), int32.
+ * Replace the __global__ kernels  apmm_w1a2 (LIB/71:80), apmm_w1a4 (LIB/78_bmmaTensorCoreGemm.cu:80),
+ * apmm_w2a2 (LIB/72_bmmaTensorCoreGemm.cu:80); w1a3 has no GEMM kernel in the reference tree (only
+ * the mirrored apmm_w3a1, LIB/79_bmmaTensorCoreGemm.cu:80) and follows the same definition.
+ * wb / xb must equal the bit widths in the function name.  Requires K % 128 == 0 (int4 rows). */
+int apmm_w1a2(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w1a3(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w1a4(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w2a2(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+
+/* Same accumulate, then the low xb bits of each result packed MSB-first along N:
+ * D:[xb][M][N/32] uint32.  Replace apmm_w1a2_decompose (LIB/66h:82-280) and apmm_w2a2_decompose
+ * (LIB/73_bmmaTensorCoreGemm.cuh:82).  Requires N % 32 == 0. */
+int apmm_w1a2_decompose(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w1a3_decompose(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w1a4_decompose(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w2a2_decompose(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+
+/* 3x3 / stride 1 / pad 1 convolution on a halo-stored input, int32 NHWC output.
+ * Replace compute_conv_imma: w1a2 LIB/51:58, w1a4 LIB/53_bmmaTensorCoreGemm.cu:58,
+ * w1a3 LIB/59_bmmaTensorCoreGemm.cu:58, w2a2 LIB/48_bmmaTensorCoreGemm.cu:58.
+ * Requires CIN % 128 == 0; any Height / Width / COUT. */
+int apconv_w1a2(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int apconv_w1a3(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int apconv_w1a4(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int apconv_w2a2(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+
+/* Convolution, then low-bit planes of the result: Output:[a][H][W][COUT/32].
+ * Replace APConv_w1a2_pack (LIB/67h:60-325) and APConv_w2a2_pack (LIB/70_bmmaTensorCoreGemm.cu:58).
+ * Requires COUT % 32 == 0. */
+int APConv_w1a2_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int APConv_w1a3_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int APConv_w1a4_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int APConv_w2a2_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+
+/* Convolution, 2x2 average pool with C integer division, then low-bit planes:
+ * Output:[a][H/2][W/2][COUT/32].  Replace APConv_w1a2_pack_pool (LIB/68_bmmaTensorCoreGemm.cu:58)
+ * and APConv_w2a2_pack_pool (LIB/69_bmmaTensorCoreGemm.cuh:60).  Requires even Height and Width. */
+int APConv_w1a2_pack_pool(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int APConv_w2a2_pack_pool(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+
+/* ---- general descriptor entry points ------------------------------------------------------- */
+
+enum { APNN_EPI_INT32 = 0,    /* int32 result                                                     */
+       APNN_EPI_LOWBITS = 1,  /* low out_bits bits of the result, packed (LIB/66h:255-276)         */
+       APNN_EPI_BN = 2 };     /* per-channel thresholds -> out_bits code, packed                   */
+enum { APNN_POOL_NONE = 0,
+       APNN_POOL_AVG2X2 = 1,  /* (v0+v1+v2+v3)/4 on the int32 result before quantizing (LIB/68:280-292) */
+       APNN_POOL_MAX2X2 = 2 };/* max over the 2x2 window of the quantized codes                     */
+enum { APNN_PATH_AUTO = 0, APNN_PATH_VALU = 1, APNN_PATH_MFMA = 2 };
+/* `path` fields: low byte = APNN_PATH_*; bits 8..15 = 0 (library picks the tile shape) or
+ * 1 + tile index to pin it (tuning / test coverage of every tile shape; APNN_EINVAL if the
+ * chosen kernel family has no such tile or the epilogue cannot use it). */
+#define APNN_PATH_TILE(path, tile) ((path) | (((tile) + 1) << 8))
+enum { APNN_WEIGHT_UNSIGNED = 0,   /* planes are an unsigned integer u (the reference's arithmetic)    */
+       APNN_WEIGHT_SYMMETRIC = 1 };/* weight value is 2u - (2^wb - 1); wb = 1 gives {-1,+1}            */
+
+/* Output stage shared by GEMM and convolution.  "channel" is the fast output index
+ * (N for GEMM, COUT for convolution).
+ *   v = acc (after AVG pooling if requested) + (residual ? residual[row][channel] : 0)
+ *   save_acc (optional) receives v as int32 [rows][channels]   (cf. save_residual, NN/kernel.cuh:779-831)
+ *   LOWBITS: code = v & (2^out_bits - 1)
+ *   BN     : code = #{ k < 2^out_bits-1 : (flip[channel] ? -v : v) >= thresholds[channel][k] }
+ *            (out_bits = 1 is the reference's  !(v < bn[channel]), NN/kernel.cuh:833-834)
+ *   planes of code are written MSB-first: [out_bits][rows][channels/32].
+ * residual / save_acc cannot be combined with pooling. */
+typedef struct apnn_epilogue {
+  int mode;                  /* APNN_EPI_* */
+  int out_bits;              /* 1..8, LOWBITS / BN */
+  int pool;                  /* APNN_POOL_*, convolution only */
+  const int32_t *thresholds; /* device, [channels][2^out_bits - 1], non-decreasing per channel (BN) */
+  const uint8_t *flip;       /* device, [channels] or NULL (BN) */
+  const int32_t *residual;   /* device, [rows][channels] int32 or NULL */
+  int32_t *save_acc;         /* device, [rows][channels] int32 or NULL */
+} apnn_epilogue;
+
+/* out[m][n] over W:[wb][M][K/32] (slow index) and X:[xb][N][K/32] (fast index). */
+typedef struct apnn_gemm_desc {
+  const void *W, *X;
+  void *D;
+  int M, N, K;               /* K % 128 == 0 */
+  int wb, xb;                /* 1..4 each */
+  int weight_mode;           /* APNN_WEIGHT_*; SYMMETRIC makes W the signed operand */
+  apnn_epilogue epi;
+  int path;                  /* APNN_PATH_* */
+} apnn_gemm_desc;
+int apnn_gemm(const apnn_gemm_desc *d, apnn_stream_t s);
+
+/* Convolution / fully-connected (R=S=1, H=W=1, batch = rows) over NHWC bit-planes.
+ * X:[xb][batch][Hs][Ws][cin_pad/32] with Hs = H + (halo ? 2*pad : 0); W:[wb][COUT][R][S][cin_pad/32];
+ * output rows are (batch, oy, ox) in raster order, channels COUT. */
+typedef struct apnn_conv_desc {
+  const void *W, *X;
+  void *O;
+  int batch, H, Wd;          /* logical input size */
+  int cin_pad;               /* stored channels per pixel, multiple of 32 (reference: multiple of 128) */
+  int COUT;
+  int R, S, stride, pad;
+  int halo;                  /* 1: input stored with its halo, whose contents take part (LIB/51:395);
+                                0: unpadded input, out-of-image taps are zero */
+  int wb, xb;
+  int weight_mode;           /* SYMMETRIC makes W the signed operand */
+  apnn_epilogue epi;
+  int path;
+} apnn_conv_desc;
+int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s);
+
+/* Bit-plane packer with the layout of Bit_compression (NN/kernel.cuh:46-77):
+ * values:[rows][C] uint32 codes -> planes:[bits][rows][cpad/32], channel c at bit 31-c%32,
+ * pad channels zero.  cpad % 32 == 0, cpad >= C. */
+int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits, apnn_stream_t s);
+
+/* Library / device information: number of compute units of the current device (0 if none). */
+int apnn_device_cus(void);
+const char *apnn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,77 @@
+"""Device-side plumbing for the GPU parity tests: torch only allocates device memory and supplies
+streams; every compute call goes through the C ABI of libapnn_tc.so."""
+import ctypes
+
+import numpy as np
+import torch
+
+import pkg
+
+A = pkg.load()
+
+
+def to_dev(arr):
+    arr = np.ascontiguousarray(arr)
+    if arr.dtype == np.uint32:
+        arr = arr.view(np.int32)
+    return torch.from_numpy(arr).cuda()
+
+
+def dev_empty_i32(n, fill=None):
+    t = torch.empty(int(n), dtype=torch.int32, device="cuda")
+    if fill is not None:
+        t.fill_(fill)
+    return t
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def to_host(t, dtype=np.int32):
+    torch.cuda.synchronize()
+    a = t.cpu().numpy()
+    return a.view(dtype) if dtype != a.dtype else a
+
+
+def epilogue(mode=0, out_bits=0, pool=0, thr=None, flip=None, resid=None, save=None):
+    e = A.Epilogue()
+    e.mode, e.out_bits, e.pool = mode, out_bits, pool
+    e.thresholds = thr.data_ptr() if thr is not None else None
+    e.flip = flip.data_ptr() if flip is not None else None
+    e.residual = resid.data_ptr() if resid is not None else None
+    e.save_acc = save.data_ptr() if save is not None else None
+    return e
+
+
+def run_gemm(W, X, M, N, K, wb, xb, *, sym=0, epi=None, path=0, tile=None, out_words=None):
+    """W, X: numpy uint32 planes.  Returns the raw int32 output buffer as numpy."""
+    dW, dX = to_dev(W), to_dev(X)
+    epi = epi or epilogue()
+    if out_words is None:
+        out_words = M * N if epi.mode == 0 else epi.out_bits * M * (N // 32)
+    out = dev_empty_i32(out_words, fill=-7)
+    d = A.GemmDesc(W=dW.data_ptr(), X=dX.data_ptr(), D=out.data_ptr(), M=M, N=N, K=K, wb=wb, xb=xb,
+                   weight_mode=sym, epi=epi, path=path if tile is None else (path | ((tile + 1) << 8)))
+    rc = A.lib().apnn_gemm(ctypes.byref(d), None)
+    A.check(rc, "apnn_gemm")
+    return to_host(out)
+
+
+def run_conv(Wt, X, *, batch, H, W, cin_pad, cout, R, S, stride, pad, halo, wb, xb, sym=0, epi=None,
+             path=0, tile=None):
+    dW, dX = to_dev(Wt), to_dev(X)
+    epi = epi or epilogue()
+    Ho, Wo = (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
+    rows = batch * Ho * Wo
+    if epi.mode == 0:
+        out_words = rows * cout
+    else:
+        out_words = epi.out_bits * (rows // 4 if epi.pool else rows) * (cout // 32)
+    out = dev_empty_i32(out_words, fill=-7)
+    d = A.ConvDesc(W=dW.data_ptr(), X=dX.data_ptr(), O=out.data_ptr(), batch=batch, H=H, Wd=W,
+                   cin_pad=cin_pad, COUT=cout, R=R, S=S, stride=stride, pad=pad, halo=halo, wb=wb, xb=xb,
+                   weight_mode=sym, epi=epi, path=path if tile is None else (path | ((tile + 1) << 8)))
+    rc = A.lib().apnn_conv(ctypes.byref(d), None)
+    A.check(rc, "apnn_conv")
+    return to_host(out)

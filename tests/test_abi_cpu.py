@@ -1,0 +1,67 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the header declares,
+and rejects out-of-contract arguments with an error code instead of aborting.  No compute calls."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import pkg
+
+A = pkg.load()
+ROOT = pkg.ROOT
+
+
+def test_library_exports_every_declared_symbol():
+    L = A.lib()
+    header = open(os.path.join(ROOT, "include", "apnn_tc.h")).read()
+    declared = set(re.findall(r"^(?:int|const char \*)\s*\*?(\w+)\(", header, flags=re.M))
+    assert declared == set(A.DECLARED_SYMBOLS), declared ^ set(A.DECLARED_SYMBOLS)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert b"gfx950" in L.apnn_version()
+
+
+def test_struct_sizes_match_header_layout():
+    # 3 ints (+pad) + 4 pointers; keeps the ctypes mirror honest about field order
+    assert ctypes.sizeof(A.Epilogue) == 16 + 4 * 8
+    assert A.GemmDesc.epi.offset == 3 * 8 + 6 * 4
+    assert A.ConvDesc.epi.offset == 3 * 8 + 13 * 4 + 4
+
+
+def test_named_entry_points_reject_bad_arguments():
+    L = A.lib()
+    good = 0x1000  # never dereferenced: every call below must fail validation first
+    assert L.apmm_w1a2(None, good, good, 64, 128, 128, 1, 2, None) == A.ENULL
+    assert L.apmm_w1a2(good, good + 4, good, 64, 128, 128, 1, 2, None) == A.EALIGN
+    assert L.apmm_w1a2(good, good, good, 64, 128, 100, 1, 2, None) == A.EINVAL      # K % 128
+    assert L.apmm_w1a2(good, good, good, 0, 128, 128, 1, 2, None) == A.EINVAL
+    assert L.apmm_w1a2(good, good, good, 64, 128, 128, 2, 2, None) == A.EINVAL      # wrong bit widths
+    assert L.apmm_w1a2_decompose(good, good, good, 64, 100, 128, 1, 2, None) == A.EINVAL  # N % 32
+    assert L.apconv_w1a2(good, good, good, 16, 16, 96, 128, None) == A.EINVAL       # CIN % 128
+    assert L.APConv_w1a2_pack(good, good, good, 16, 16, 128, 100, None) == A.EINVAL  # COUT % 32
+    assert L.APConv_w1a2_pack_pool(good, good, good, 15, 16, 128, 128, None) == A.EINVAL  # odd height
+    assert L.apnn_pack_bits(None, good, 4, 64, 128, 2, None) == A.ENULL
+    assert L.apnn_pack_bits(good, good, 4, 200, 128, 2, None) == A.EINVAL
+
+
+def test_descriptor_entry_points_reject_bad_arguments():
+    L = A.lib()
+    good = 0x1000
+    assert L.apnn_gemm(None, None) == A.ENULL
+    d = A.GemmDesc(W=good, X=good, D=good, M=64, N=128, K=128, wb=1, xb=2)
+    d.epi.mode = 7
+    assert L.apnn_gemm(ctypes.byref(d), None) == A.EINVAL
+    d.epi.mode = A.EPI_BN
+    d.epi.out_bits = 2
+    assert L.apnn_gemm(ctypes.byref(d), None) == A.ENULL                            # thresholds missing
+    d.epi.mode = A.EPI_INT32
+    d.epi.pool = A.POOL_AVG2X2
+    assert L.apnn_gemm(ctypes.byref(d), None) == A.EINVAL                           # pooling is conv-only
+    c = A.ConvDesc(W=good, X=good, O=good, batch=1, H=8, Wd=8, cin_pad=48, COUT=64, R=3, S=3,
+                   stride=1, pad=1, wb=1, xb=2)
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EINVAL                           # cin_pad % 32
+    c.cin_pad = 64
+    c.R = 11
+    c.pad = 0
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EINVAL                           # filter larger than image

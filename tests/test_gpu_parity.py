@@ -1,0 +1,275 @@
+"""GPU parity: libapnn_tc.so (through its C ABI) against the CPU oracle and the committed golden
+fixtures.  Integer work, so every comparison is bit-exact."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+COMBOS = [(1, 2), (1, 3), (1, 4), (2, 2)]          # (weight bits, activation bits)
+NAMES = {(1, 2): "w1a2", (1, 3): "w1a3", (1, 4): "w1a4", (2, 2): "w2a2"}
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    return gpu_util
+
+
+def _golden():
+    return np.load(os.path.join(O.GOLDEN_DIR, "golden_outputs.npz"), allow_pickle=False)
+
+
+# ---- GEMM ------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+def test_gemm_named_entry_golden(G, wb, xb):
+    """Reference-derived known answers through the reference's own entry-point names."""
+    name = NAMES[(wb, xb)]
+    M, N, K = 64, 128, 128
+    s = O.golden_stream()
+    nw, nx = wb * M * K // 32, xb * N * K // 32
+    dW, dX = G.to_dev(s[:nw]), G.to_dev(s[nw:nw + nx])
+    out = G.dev_empty_i32(M * N, fill=-7)
+    fn = getattr(G.A.lib(), "apmm_" + name)
+    G.A.check(fn(G.ptr(dW), G.ptr(dX), G.ptr(out), M, N, K, wb, xb, None), name)
+    got = G.to_host(out).reshape(M, N)
+    assert np.array_equal(got, _golden()["gemm_" + name])
+    # decompose: low xb bits, MSB-first
+    outp = G.dev_empty_i32(xb * M * N // 32, fill=-7)
+    fn = getattr(G.A.lib(), "apmm_" + name + "_decompose")
+    G.A.check(fn(G.ptr(dW), G.ptr(dX), G.ptr(outp), M, N, K, wb, xb, None), name)
+    gotp = G.to_host(outp, np.uint32).reshape(xb, M, N // 32)
+    assert np.array_equal(gotp, O.lowbits_pack(_golden()["gemm_" + name], M, N, xb))
+
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("nk", [128, 256, 384, 512, 640, 768, 896, 1024])
+def test_gemm_sweep_m64(G, wb, xb, nk):
+    """The benchmark sweep of the reference: M=64, N=K=128..1024 (LIB/78_bmmaTensorCoreGemm.cu:473-477)."""
+    rng = np.random.default_rng(1000 + nk + 7 * wb + xb)
+    M, N, K = 64, nk, nk
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb).reshape(M, N)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, nthreads=8))
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("wb,xb", COMBOS)
+def test_gemm_every_tile_ragged(G, wb, xb, tile):
+    """Row / column counts that are not multiples of any tile, every tile shape pinned."""
+    rng = np.random.default_rng(50 + tile + 10 * wb + xb)
+    M, N, K = 70, 97, 384
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, path=G.A.PATH_VALU, tile=tile).reshape(M, N)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 128), (1, 32, 128), (3, 5, 256), (64, 32, 128), (129, 64, 2048)])
+def test_gemm_edge_shapes(G, M, N, K):
+    rng = np.random.default_rng(M * 1000 + N)
+    W = O.random_planes(rng, 1, M, K // 32)
+    X = O.random_planes(rng, 2, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, 1, 2).reshape(M, N)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, 1, 2))
+
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+def test_gemm_symmetric_weights(G, wb, xb):
+    rng = np.random.default_rng(77 + wb + xb)
+    M, N, K = 64, 256, 512
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1).reshape(M, N)
+    expect = (2 * O.unpack_planes_lsb(W) - (2 ** wb - 1)) @ O.unpack_planes_lsb(X).T
+    assert np.array_equal(got, expect)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=1))
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_gemm_bn_epilogue_with_residual(G, tile):
+    rng = np.random.default_rng(91 + tile)
+    M, N, K, wb, xb, ob = 48, 160, 256, 1, 2, 2
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, wb, xb, sym_w=1)
+    resid = rng.integers(-40, 40, size=(M, N)).astype(np.int32)
+    thr = np.sort(rng.integers(-120, 120, size=(N, 2 ** ob - 1)), axis=1).astype(np.int32)
+    flip = rng.integers(0, 2, size=N).astype(np.uint8)
+    d_thr, d_flip, d_res = G.to_dev(thr), G.to_dev(flip), G.to_dev(resid)
+    d_save = G.dev_empty_i32(M * N, fill=-7)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, flip=d_flip, resid=d_res, save=d_save)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1, epi=epi, tile=tile).view(np.uint32).reshape(ob, M, N // 32)
+    q = O.bn_quantize(acc, resid, thr, flip, ob)
+    assert np.array_equal(got, O.lowbits_pack(q, M, N, ob))
+    assert np.array_equal(G.to_host(d_save).reshape(M, N), acc + resid)
+
+
+# ---- convolution -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+def test_conv_named_entry_golden(G, wb, xb):
+    name = NAMES[(wb, xb)]
+    H = Wd = 16
+    CIN = COUT = 128
+    s = O.golden_stream()
+    nx, nw = xb * (H + 2) * (Wd + 2) * CIN // 32, wb * COUT * 9 * CIN // 32
+    dX, dW = G.to_dev(s[:nx]), G.to_dev(s[nx:nx + nw])
+    out = G.dev_empty_i32(H * Wd * COUT, fill=-7)
+    L = G.A.lib()
+    G.A.check(getattr(L, "apconv_" + name)(G.ptr(dW), G.ptr(dX), G.ptr(out), H, Wd, CIN, COUT, None), name)
+    gold = _golden()
+    assert np.array_equal(G.to_host(out).reshape(H, Wd, COUT), gold["conv_" + name])
+    outp = G.dev_empty_i32(xb * H * Wd * COUT // 32, fill=-7)
+    G.A.check(getattr(L, "APConv_" + name + "_pack")(G.ptr(dW), G.ptr(dX), G.ptr(outp), H, Wd, CIN, COUT, None), name)
+    assert np.array_equal(G.to_host(outp, np.uint32).reshape(xb, H * Wd, COUT // 32), gold["conv_pack_" + name])
+    if name in ("w1a2", "w2a2"):
+        outq = G.dev_empty_i32(xb * (H // 2) * (Wd // 2) * COUT // 32, fill=-7)
+        G.A.check(getattr(L, "APConv_" + name + "_pack_pool")(G.ptr(dW), G.ptr(dX), G.ptr(outq), H, Wd, CIN, COUT, None), name)
+        pooled = O.avgpool2x2(gold["conv_" + name][None])[0]
+        expect = O.lowbits_pack(pooled, (H // 2) * (Wd // 2), COUT, xb)
+        assert np.array_equal(G.to_host(outq, np.uint32).reshape(expect.shape), expect)
+
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("C,batch", [(128, 1), (256, 1), (512, 1), (128, 16)])
+def test_conv3x3_16x16_sweep(G, wb, xb, C, batch):
+    """Benchmark family of the reference: 3x3 / stride 1 / pad 1 on a 16x16 map, halo stored."""
+    rng = np.random.default_rng(300 + C + batch + wb * 3 + xb)
+    H = Wd = 16
+    X = O.random_planes(rng, xb, batch * (H + 2) * (Wd + 2), C // 32)
+    Wt = O.random_planes(rng, wb, C * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=1, wb=wb, xb=xb)
+    got = G.run_conv(Wt, X, cin_pad=C, **kw).reshape(batch, H, Wd, C)
+    assert np.array_equal(got, O.conv(Wt, X, cwords=C // 32, nthreads=8, **kw))
+
+
+GEOMS = [  # batch H W cin_pad cout R stride pad halo
+    (2, 14, 14, 128, 96, 3, 1, 1, 0),     # predicated halo, cout not a tile multiple
+    (3, 28, 28, 64, 128, 3, 2, 1, 0),     # ResNet stride-2 3x3 on 64 stored channels (64-bit loads)
+    (2, 28, 28, 64, 128, 1, 2, 0, 0),     # ResNet 1x1 stride-2 downsample
+    (1, 7, 7, 256, 64, 3, 1, 1, 0),       # 7x7 map
+    (2, 13, 11, 32, 40, 5, 1, 2, 0),      # 5x5 filter, 32 stored channels (32-bit loads)
+    (8, 1, 1, 512, 256, 1, 1, 0, 0),      # fully connected layer as 1x1 conv, batch = rows
+    (1, 9, 9, 128, 32, 3, 1, 1, 1),       # halo stored, odd size
+]
+
+
+@pytest.mark.parametrize("geom", GEOMS)
+@pytest.mark.parametrize("wb,xb,sym", [(1, 2, 0), (1, 2, 1), (2, 2, 1), (1, 4, 0), (1, 3, 1)])
+def test_conv_general_geometry(G, geom, wb, xb, sym):
+    batch, H, Wd, cin_pad, cout, R, stride, pad, halo = geom
+    rng = np.random.default_rng(hash((geom, wb, xb, sym)) % (2 ** 31))
+    Hs, Ws = (H + 2 * pad, Wd + 2 * pad) if halo else (H, Wd)
+    X = O.random_planes(rng, xb, batch * Hs * Ws, cin_pad // 32)
+    Wt = O.random_planes(rng, wb, cout * R * R, cin_pad // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=R, S=R, stride=stride, pad=pad, halo=halo, wb=wb, xb=xb)
+    expect = O.conv(Wt, X, cwords=cin_pad // 32, sym_w=sym, nthreads=8, **kw)
+    got = G.run_conv(Wt, X, cin_pad=cin_pad, sym=sym, **kw).reshape(expect.shape)
+    assert np.array_equal(got, expect)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+def test_conv_every_tile(G, tile):
+    rng = np.random.default_rng(400 + tile)
+    batch, H, Wd, C, cout = 2, 10, 6, 128, 72
+    X = O.random_planes(rng, 2, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, 1, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=1, xb=2)
+    expect = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, path=G.A.PATH_VALU, tile=tile, **kw).reshape(expect.shape)
+    assert np.array_equal(got, expect)
+
+
+@pytest.mark.parametrize("pool", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_conv_bn_epilogue(G, pool, tile):
+    """BN-threshold requantize to a bits (+ residual / saved accumulator when not pooling,
+    + avg / max pooling), packed for the next layer."""
+    rng = np.random.default_rng(500 + 10 * pool + tile)
+    batch, H, Wd, C, cout, wb, xb, ob = 2, 8, 12, 128, 96, 1, 2, 2
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw)
+    thr = np.sort(rng.integers(-300, 300, size=(cout, 2 ** ob - 1)), axis=1).astype(np.int32)
+    flip = rng.integers(0, 2, size=cout).astype(np.uint8)
+    d_thr, d_flip = G.to_dev(thr), G.to_dev(flip)
+    if pool == 0:
+        resid = rng.integers(-100, 100, size=acc.shape).astype(np.int32)
+        d_res, d_save = G.to_dev(resid), G.dev_empty_i32(acc.size, fill=-7)
+        epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, flip=d_flip, resid=d_res, save=d_save)
+        q = O.bn_quantize(acc.reshape(-1, cout), resid.reshape(-1, cout), thr, flip, ob)
+        rows = batch * H * Wd
+    else:
+        epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, pool=pool, thr=d_thr, flip=d_flip)
+        if pool == 1:
+            q = O.bn_quantize(O.avgpool2x2(acc).reshape(-1, cout), None, thr, flip, ob)
+        else:
+            q = O.maxpool2x2(O.bn_quantize(acc.reshape(-1, cout), None, thr, flip, ob).reshape(acc.shape)).reshape(-1, cout)
+        rows = batch * (H // 2) * (Wd // 2)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, tile=tile, **kw).view(np.uint32).reshape(ob, rows, cout // 32)
+    assert np.array_equal(got, O.lowbits_pack(q, rows, cout, ob))
+    if pool == 0:
+        assert np.array_equal(G.to_host(d_save).reshape(acc.shape), acc + resid)
+
+
+def test_packed_output_feeds_next_layer(G):
+    """A layer's packed output is a valid activation operand of the next layer: unpacking it with the
+    packer's bit order (MSB-first) reproduces the codes, and a GEMM on it matches the oracle."""
+    rng = np.random.default_rng(600)
+    batch, C, cout, nxt = 16, 256, 128, 64
+    X = O.random_planes(rng, 2, batch, C // 32)
+    Wt = O.random_planes(rng, 1, cout, C // 32)
+    kw = dict(batch=batch, H=1, W=1, cout=cout, R=1, S=1, stride=1, pad=0, halo=0, wb=1, xb=2)
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw).reshape(batch, cout)
+    thr = np.sort(rng.integers(-60, 60, size=(cout, 3)), axis=1).astype(np.int32)
+    d_thr = G.to_dev(thr)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=2, thr=d_thr)
+    packed = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, **kw).view(np.uint32).reshape(2, batch, cout // 32)
+    q = O.bn_quantize(acc, None, thr, None, 2)
+    assert np.array_equal(O.unpack_bits(packed, batch, cout, cout, 2), q.astype(np.uint32))
+    W2 = O.random_planes(rng, 1, nxt, cout // 32)
+    kw2 = dict(batch=batch, H=1, W=1, cout=nxt, R=1, S=1, stride=1, pad=0, halo=0, wb=1, xb=2)
+    got = G.run_conv(W2, packed, cin_pad=cout, **kw2).reshape(batch, nxt)
+    assert np.array_equal(got, O.conv(W2, packed, cwords=cout // 32, **kw2).reshape(batch, nxt))
+
+
+def test_pack_bits(G):
+    rng = np.random.default_rng(700)
+    for rows, C, cpad, bits in [(5, 3, 128, 2), (33, 70, 128, 3), (64, 192, 256, 2), (7, 64, 64, 8), (2, 100, 128, 1)]:
+        v = rng.integers(0, 2 ** bits, size=(rows, C)).astype(np.uint32)
+        dv = G.to_dev(v)
+        out = G.dev_empty_i32(bits * rows * cpad // 32, fill=-7)
+        G.A.check(G.A.lib().apnn_pack_bits(G.ptr(dv), G.ptr(out), rows, C, cpad, bits, None), "pack_bits")
+        got = G.to_host(out, np.uint32).reshape(bits, rows, cpad // 32)
+        assert np.array_equal(got, O.pack_bits(v, rows, C, cpad, bits))
+
+
+# ---- full-size shapes: size-independent properties + sampled rows ------------------------------
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+def test_gemm_2048_sampled_and_closed_form(G, wb, xb):
+    rng = np.random.default_rng(800 + wb + xb)
+    M = N = K = 2048
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb).reshape(M, N)
+    rows = np.sort(rng.choice(M, 16, replace=False))
+    for m in rows:
+        assert np.array_equal(got[m], O.gemm_rows(W, X, M, N, K, wb, xb, int(m), int(m) + 1, nthreads=8)[0])
+    # column sums are linear in W:  sum_m D[m][n] = (sum_m wvalue[m]) . xvalue[n]
+    wsum = O.unpack_planes_lsb(W).sum(0)
+    assert np.array_equal(got.astype(np.int64).sum(0), O.unpack_planes_lsb(X) @ wsum)
+    ones_w = np.full_like(W, 0xFFFFFFFF)
+    ones_x = np.full_like(X, 0xFFFFFFFF)
+    assert np.all(G.run_gemm(ones_w, ones_x, M, N, K, wb, xb) == K * (2 ** wb - 1) * (2 ** xb - 1))
