@@ -79,6 +79,12 @@ def lib():
     """The loaded library.  Raises if it has not been built: there is no fallback path."""
     global _lib
     if _lib is None:
+        # When PyTorch supplies the device buffers, its bundled HIP runtime has to be the one this
+        # library binds to (same SONAME): two runtimes in one process do not share allocations.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         if not os.path.exists(LIB_PATH):
             raise ApnnError("%s is missing: run `make -C apnn-tc_amd/csrc` (or __graft_entry__.build())" % LIB_PATH)
         L = ctypes.CDLL(LIB_PATH)

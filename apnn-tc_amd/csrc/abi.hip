@@ -89,6 +89,53 @@ void fill_epilogue(KParams &p, const apnn_epilogue &e, void *out, long long out_
 
 typedef hipError_t (*valu_fn)(int, int, const KParams &, hipStream_t);
 
+valu_fn mfma_gemm_fn(int wb, int xb) {
+  if (wb == 1 && xb == 2) return apnn::mfma_gemm_1_2_x;
+  if (wb == 1 && xb == 3) return apnn::mfma_gemm_1_3_x;
+  if (wb == 1 && xb == 4) return apnn::mfma_gemm_1_4_x;
+  if (wb == 2 && xb == 2) return apnn::mfma_gemm_2_2_x;
+  return nullptr;
+}
+
+valu_fn mfma_conv_fn(int xb, int wb) {
+  if (xb == 2 && wb == 1) return apnn::mfma_conv_2_1_x;
+  if (xb == 3 && wb == 1) return apnn::mfma_conv_3_1_x;
+  if (xb == 4 && wb == 1) return apnn::mfma_conv_4_1_x;
+  if (xb == 2 && wb == 2) return apnn::mfma_conv_2_2_x;
+  return nullptr;
+}
+
+// MFMA tile: largest shape that still yields one work-group per compute unit; narrow outputs
+// (<= 64 channels) take the 128x64 shape; otherwise the smallest.
+int choose_mfma_tile(int rowsA, int rowsB) {
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;
+  auto ntiles = [&](int t) {
+    return (long long)((rowsA + apnn::kMfmaTileA[t] - 1) / apnn::kMfmaTileA[t]) *
+           ((rowsB + apnn::kMfmaTileB[t] - 1) / apnn::kMfmaTileB[t]);
+  };
+  if (rowsB <= 64) return ntiles(3) >= cus ? 3 : 2;
+  for (int t = 0; t < 2; ++t)
+    if (ntiles(t) >= cus) return t;
+  return 2;
+}
+
+int pick_mfma_tile(int tile_pin, const KParams &p, int *tile) {
+  if (tile_pin == 0) {
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB);
+    return APNN_OK;
+  }
+  if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
+  *tile = tile_pin - 1;
+  return APNN_OK;
+}
+
+// AUTO: the matrix-core path pays off once every wave has full 32x32 blocks to fill and the
+// reduction is long enough to amortise the epilogue; small problems stay on the VALU path.
+bool auto_prefers_mfma(const KParams &p) {
+  return (long long)p.rowsA * p.rowsB >= 256LL * 256 && p.KW >= 8;
+}
+
 valu_fn valu_gemm_fn(int wb, int xb) {
   if (wb == 1 && xb == 2) return apnn::valu_gemm_1_2_x;
   if (wb == 1 && xb == 3) return apnn::valu_gemm_1_3_x;
@@ -129,10 +176,15 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   p.wmax = (1 << d->wb) - 1;
   fill_epilogue(p, d->epi, d->D, d->M);
 
-  if (path == APNN_PATH_MFMA) return APNN_EUNSUPPORTED;
+  int tile;
+  if (path == APNN_PATH_MFMA || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+    valu_fn fn = mfma_gemm_fn(d->wb, d->xb);
+    if (fn == nullptr) return APNN_EUNSUPPORTED;
+    if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
+    return (int)fn(4, tile, p, stream);
+  }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
-  int tile;
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
   return (int)fn(4, tile, p, stream);
 }
@@ -183,10 +235,15 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   p.wmax = (1 << d->wb) - 1;
   fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
 
-  if (path == APNN_PATH_MFMA) return APNN_EUNSUPPORTED;
+  int tile;
+  if (path == APNN_PATH_MFMA || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+    valu_fn fn = mfma_conv_fn(d->xb, d->wb);
+    if (fn == nullptr) return APNN_EUNSUPPORTED;
+    if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
+    return (int)fn(vw, tile, p, stream);
+  }
   valu_fn fn = valu_conv_fn(d->xb, d->wb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
-  int tile;
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
   return (int)fn(vw, tile, p, stream);
 }

@@ -71,4 +71,20 @@ int apnn_bench_empty(int warmup, int iters, apnn_stream_t s, float *event_ms, do
       warmup, iters, stream, event_ms, wall_ms);
 }
 
+__global__ __launch_bounds__(256) void apnn_bench_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                              long long n16) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16;
+       i += (long long)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+// Plain device-to-device copy of `bytes` (multiple of 16): reads `bytes`, writes `bytes`.  Used to
+// calibrate the HBM traffic counters (FETCH_SIZE / WRITE_SIZE) against a kernel of known traffic.
+int apnn_bench_copy(const void *src, void *dst, long long bytes, apnn_stream_t s) {
+  if (src == nullptr || dst == nullptr || bytes <= 0 || (bytes % 16) != 0) return APNN_EINVAL;
+  hipLaunchKernelGGL(apnn_bench_copy_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(s),
+                     static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), bytes / 16);
+  return (int)hipGetLastError();
+}
+
 }  // extern "C"

@@ -18,6 +18,23 @@ APNN_DECL_VALU(conv, 4, 1)
 APNN_DECL_VALU(conv, 2, 2)
 #undef APNN_DECL_VALU
 
+#define APNN_DECL_MFMA(kind, pa, pb) \
+  hipError_t mfma_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);
+APNN_DECL_MFMA(gemm, 1, 2)
+APNN_DECL_MFMA(gemm, 1, 3)
+APNN_DECL_MFMA(gemm, 1, 4)
+APNN_DECL_MFMA(gemm, 2, 2)
+APNN_DECL_MFMA(conv, 2, 1)
+APNN_DECL_MFMA(conv, 3, 1)
+APNN_DECL_MFMA(conv, 4, 1)
+APNN_DECL_MFMA(conv, 2, 2)
+#undef APNN_DECL_MFMA
+
+// tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
+constexpr int kMfmaTileCount = 4;
+constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128};
+constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64};
+
 // aux_kernels.hip
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
                             hipStream_t s);

@@ -40,6 +40,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also launch one 256 MiB device copy (known traffic) for counter calibration")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -88,6 +90,14 @@ def main():
                 ref = O.gemm_rows(W, X, M, N, K, wb, xb, m, m + 1, sym_w=sym, nthreads=os.cpu_count() or 1)[0]
                 ok = ok and bool(np.array_equal(got[m], ref))
         return dict(event_ms=ev.value / iters, wall_ms=wall.value / iters, verified=ok, W=W, X=X)
+
+    if args.copy_calib:
+        nbytes_c = 256 << 20
+        src = torch.zeros(nbytes_c // 4, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        benchlib.apnn_bench_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p]
+        A.check(benchlib.apnn_bench_copy(src.data_ptr(), dst.data_ptr(), nbytes_c, stream), "apnn_bench_copy")
+        torch.cuda.synchronize()
 
     # ---- headline -----------------------------------------------------------------------------
     M, N, K, wb, xb = 64, 1024, 1024, 1, 2

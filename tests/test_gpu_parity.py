@@ -50,53 +50,60 @@ def test_gemm_named_entry_golden(G, wb, xb):
     assert np.array_equal(gotp, O.lowbits_pack(_golden()["gemm_" + name], M, N, xb))
 
 
+PATHS = [1, 2]   # APNN_PATH_VALU, APNN_PATH_MFMA
+
+
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("wb,xb", COMBOS)
 @pytest.mark.parametrize("nk", [128, 256, 384, 512, 640, 768, 896, 1024])
-def test_gemm_sweep_m64(G, wb, xb, nk):
+def test_gemm_sweep_m64(G, wb, xb, nk, path):
     """The benchmark sweep of the reference: M=64, N=K=128..1024 (LIB/78_bmmaTensorCoreGemm.cu:473-477)."""
     rng = np.random.default_rng(1000 + nk + 7 * wb + xb)
     M, N, K = 64, nk, nk
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, wb, xb).reshape(M, N)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, path=path).reshape(M, N)
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, nthreads=8))
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("tile", [0, 1, 2, 3])
 @pytest.mark.parametrize("wb,xb", COMBOS)
-def test_gemm_every_tile_ragged(G, wb, xb, tile):
+def test_gemm_every_tile_ragged(G, wb, xb, tile, path):
     """Row / column counts that are not multiples of any tile, every tile shape pinned."""
     rng = np.random.default_rng(50 + tile + 10 * wb + xb)
-    M, N, K = 70, 97, 384
+    M, N, K = (70, 97, 384) if path == 1 else (300, 289, 640)
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, wb, xb, path=G.A.PATH_VALU, tile=tile).reshape(M, N)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, path=path, tile=tile).reshape(M, N)
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb))
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("M,N,K", [(1, 1, 128), (1, 32, 128), (3, 5, 256), (64, 32, 128), (129, 64, 2048)])
-def test_gemm_edge_shapes(G, M, N, K):
+def test_gemm_edge_shapes(G, M, N, K, path):
     rng = np.random.default_rng(M * 1000 + N)
     W = O.random_planes(rng, 1, M, K // 32)
     X = O.random_planes(rng, 2, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, 1, 2).reshape(M, N)
+    got = G.run_gemm(W, X, M, N, K, 1, 2, path=path).reshape(M, N)
     assert np.array_equal(got, O.gemm(W, X, M, N, K, 1, 2))
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("wb,xb", COMBOS)
-def test_gemm_symmetric_weights(G, wb, xb):
+def test_gemm_symmetric_weights(G, wb, xb, path):
     rng = np.random.default_rng(77 + wb + xb)
     M, N, K = 64, 256, 512
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1).reshape(M, N)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1, path=path).reshape(M, N)
     expect = (2 * O.unpack_planes_lsb(W) - (2 ** wb - 1)) @ O.unpack_planes_lsb(X).T
     assert np.array_equal(got, expect)
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=1))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
-def test_gemm_bn_epilogue_with_residual(G, tile):
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3)])
+def test_gemm_bn_epilogue_with_residual(G, tile, path):
     rng = np.random.default_rng(91 + tile)
     M, N, K, wb, xb, ob = 48, 160, 256, 1, 2, 2
     W = O.random_planes(rng, wb, M, K // 32)
@@ -108,7 +115,7 @@ def test_gemm_bn_epilogue_with_residual(G, tile):
     d_thr, d_flip, d_res = G.to_dev(thr), G.to_dev(flip), G.to_dev(resid)
     d_save = G.dev_empty_i32(M * N, fill=-7)
     epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, flip=d_flip, resid=d_res, save=d_save)
-    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1, epi=epi, tile=tile).view(np.uint32).reshape(ob, M, N // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1, epi=epi, path=path, tile=tile).view(np.uint32).reshape(ob, M, N // 32)
     q = O.bn_quantize(acc, resid, thr, flip, ob)
     assert np.array_equal(got, O.lowbits_pack(q, M, N, ob))
     assert np.array_equal(G.to_host(d_save).reshape(M, N), acc + resid)
@@ -140,16 +147,17 @@ def test_conv_named_entry_golden(G, wb, xb):
         assert np.array_equal(G.to_host(outq, np.uint32).reshape(expect.shape), expect)
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("wb,xb", COMBOS)
 @pytest.mark.parametrize("C,batch", [(128, 1), (256, 1), (512, 1), (128, 16)])
-def test_conv3x3_16x16_sweep(G, wb, xb, C, batch):
+def test_conv3x3_16x16_sweep(G, wb, xb, C, batch, path):
     """Benchmark family of the reference: 3x3 / stride 1 / pad 1 on a 16x16 map, halo stored."""
     rng = np.random.default_rng(300 + C + batch + wb * 3 + xb)
     H = Wd = 16
     X = O.random_planes(rng, xb, batch * (H + 2) * (Wd + 2), C // 32)
     Wt = O.random_planes(rng, wb, C * 9, C // 32)
     kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=1, wb=wb, xb=xb)
-    got = G.run_conv(Wt, X, cin_pad=C, **kw).reshape(batch, H, Wd, C)
+    got = G.run_conv(Wt, X, cin_pad=C, path=path, **kw).reshape(batch, H, Wd, C)
     assert np.array_equal(got, O.conv(Wt, X, cwords=C // 32, nthreads=8, **kw))
 
 
@@ -164,9 +172,10 @@ GEOMS = [  # batch H W cin_pad cout R stride pad halo
 ]
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("geom", GEOMS)
 @pytest.mark.parametrize("wb,xb,sym", [(1, 2, 0), (1, 2, 1), (2, 2, 1), (1, 4, 0), (1, 3, 1)])
-def test_conv_general_geometry(G, geom, wb, xb, sym):
+def test_conv_general_geometry(G, geom, wb, xb, sym, path):
     batch, H, Wd, cin_pad, cout, R, stride, pad, halo = geom
     rng = np.random.default_rng(hash((geom, wb, xb, sym)) % (2 ** 31))
     Hs, Ws = (H + 2 * pad, Wd + 2 * pad) if halo else (H, Wd)
@@ -174,25 +183,26 @@ def test_conv_general_geometry(G, geom, wb, xb, sym):
     Wt = O.random_planes(rng, wb, cout * R * R, cin_pad // 32)
     kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=R, S=R, stride=stride, pad=pad, halo=halo, wb=wb, xb=xb)
     expect = O.conv(Wt, X, cwords=cin_pad // 32, sym_w=sym, nthreads=8, **kw)
-    got = G.run_conv(Wt, X, cin_pad=cin_pad, sym=sym, **kw).reshape(expect.shape)
+    got = G.run_conv(Wt, X, cin_pad=cin_pad, sym=sym, path=path, **kw).reshape(expect.shape)
     assert np.array_equal(got, expect)
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("tile", [0, 1, 2, 3])
-def test_conv_every_tile(G, tile):
+def test_conv_every_tile(G, tile, path):
     rng = np.random.default_rng(400 + tile)
     batch, H, Wd, C, cout = 2, 10, 6, 128, 72
     X = O.random_planes(rng, 2, batch * H * Wd, C // 32)
     Wt = O.random_planes(rng, 1, cout * 9, C // 32)
     kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=1, xb=2)
     expect = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw)
-    got = G.run_conv(Wt, X, cin_pad=C, sym=1, path=G.A.PATH_VALU, tile=tile, **kw).reshape(expect.shape)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, path=path, tile=tile, **kw).reshape(expect.shape)
     assert np.array_equal(got, expect)
 
 
 @pytest.mark.parametrize("pool", [0, 1, 2])
-@pytest.mark.parametrize("tile", [0, 1, 2])
-def test_conv_bn_epilogue(G, pool, tile):
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3)])
+def test_conv_bn_epilogue(G, pool, tile, path):
     """BN-threshold requantize to a bits (+ residual / saved accumulator when not pooling,
     + avg / max pooling), packed for the next layer."""
     rng = np.random.default_rng(500 + 10 * pool + tile)
@@ -217,7 +227,7 @@ def test_conv_bn_epilogue(G, pool, tile):
         else:
             q = O.maxpool2x2(O.bn_quantize(acc.reshape(-1, cout), None, thr, flip, ob).reshape(acc.shape)).reshape(-1, cout)
         rows = batch * (H // 2) * (Wd // 2)
-    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, tile=tile, **kw).view(np.uint32).reshape(ob, rows, cout // 32)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(ob, rows, cout // 32)
     assert np.array_equal(got, O.lowbits_pack(q, rows, cout, ob))
     if pool == 0:
         assert np.array_equal(G.to_host(d_save).reshape(acc.shape), acc + resid)
@@ -257,13 +267,14 @@ def test_pack_bits(G):
 
 # ---- full-size shapes: size-independent properties + sampled rows ------------------------------
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("wb,xb", COMBOS)
-def test_gemm_2048_sampled_and_closed_form(G, wb, xb):
+def test_gemm_2048_sampled_and_closed_form(G, wb, xb, path):
     rng = np.random.default_rng(800 + wb + xb)
     M = N = K = 2048
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, wb, xb).reshape(M, N)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, path=path).reshape(M, N)
     rows = np.sort(rng.choice(M, 16, replace=False))
     for m in rows:
         assert np.array_equal(got[m], O.gemm_rows(W, X, M, N, K, wb, xb, int(m), int(m) + 1, nthreads=8)[0])
@@ -272,4 +283,4 @@ def test_gemm_2048_sampled_and_closed_form(G, wb, xb):
     assert np.array_equal(got.astype(np.int64).sum(0), O.unpack_planes_lsb(X) @ wsum)
     ones_w = np.full_like(W, 0xFFFFFFFF)
     ones_x = np.full_like(X, 0xFFFFFFFF)
-    assert np.all(G.run_gemm(ones_w, ones_x, M, N, K, wb, xb) == K * (2 ** wb - 1) * (2 ** xb - 1))
+    assert np.all(G.run_gemm(ones_w, ones_x, M, N, K, wb, xb, path=path) == K * (2 ** wb - 1) * (2 ** xb - 1))
