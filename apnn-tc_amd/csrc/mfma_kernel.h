@@ -22,6 +22,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "epilogue.h"
 #include "kparams.h"
 #include "valu_kernel.h"  // load_words, fast_div
@@ -45,6 +47,86 @@ __device__ __forceinline__ v4i expand_planes(const uint32_t (&w)[P], const uint3
     out[t] = (int)word;
   }
   return out;
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Output stage for one 32x32 accumulator block.  Register r of the block holds
+// row 8*(r/4) + 4*g + (r%4), column li (g = lane / 32, li = lane % 32).
+// ssum: activation sum of row li of this block (CONV) or of column li (GEMM entry points).
+template <bool CONV>
+__device__ __forceinline__ void mfma_epilogue_block(const KParams &p, const v16i &blk, int ssum, int rbase,
+                                                    int gcol, int g, int li) {
+  const bool col_ok = gcol < p.rowsB;
+  const int w32 = p.rowsB >> 5;
+  int v[16];
+  static_for<0, 16>([&](auto rc) {
+    constexpr int r = decltype(rc)::value;
+    int t = blk[r];
+    if (p.sym) {
+      const int rin = 8 * (r >> 2) + 4 * g + (r & 3);
+      const int s = CONV ? __shfl(ssum, rin, 64) : ssum;
+      t = 2 * t - p.wmax * s;
+    }
+    v[r] = t;
+  });
+  if (p.epi == APNN_EPI_INT32) {
+    int *out = reinterpret_cast<int *>(p.out);
+    static_for<0, 16>([&](auto rc) {
+      constexpr int r = decltype(rc)::value;
+      const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
+      if (col_ok && grow < p.rowsA) out[(long long)grow * p.rowsB + gcol] = v[r];
+    });
+  } else if (p.pool == APNN_POOL_NONE) {
+    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+    static_for<0, 16>([&](auto rc) {
+      constexpr int r = decltype(rc)::value;
+      const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
+      const bool ok = col_ok && grow < p.rowsA;
+      int code = 0;
+      if (ok) {
+        int t = v[r];
+        const long long o = (long long)grow * p.rowsB + gcol;
+        if (p.resid != nullptr) t += p.resid[o];
+        if (p.save_acc != nullptr) p.save_acc[o] = t;
+        code = quantize_code(p, t, gcol);
+      }
+      for (int b = 0; b < p.out_bits; ++b) {
+        const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
+        const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
+        if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
+      }
+    });
+  } else {
+    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+    const int out_rows_total = p.rowsA / 4;
+    static_for<0, 4>([&](auto qc) {
+      constexpr int q = decltype(qc)::value;
+      const int grow = (rbase + 8 * q + 4 * g) >> 2;  // 2x2 window index
+      const bool ok = col_ok && grow < out_rows_total;
+      int code = 0;
+      if (ok) {
+        if (p.pool == APNN_POOL_AVG2X2) {
+          code = quantize_code(p, (v[4 * q] + v[4 * q + 1] + v[4 * q + 2] + v[4 * q + 3]) / 4, gcol);
+        } else {
+          const int c0 = quantize_code(p, v[4 * q], gcol), c1 = quantize_code(p, v[4 * q + 1], gcol);
+          const int c2 = quantize_code(p, v[4 * q + 2], gcol), c3 = quantize_code(p, v[4 * q + 3], gcol);
+          code = max(max(c0, c1), max(c2, c3));
+        }
+      }
+      for (int b = 0; b < p.out_bits; ++b) {
+        const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
+        const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
+        if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
+      }
+    });
+  }
 }
 
 template <int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV>
@@ -175,11 +257,15 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[x][y][r] = 0;
 
-  // activation row sums for the symmetric-weight correction (activations: A for conv, B for GEMM)
+  // activation row sums per plane for the symmetric-weight correction (activations: A for conv,
+  // B for the GEMM entry points); always accumulated -- one popcount-accumulate per plane and
+  // fragment is cheaper than a branch that would split the k-step into basic blocks
   constexpr int FS = CONV ? FA : FB, PS = CONV ? PA : PB;
-  int ssum[FS];
+  int psum[FS][PS];
 #pragma unroll
-  for (int x = 0; x < FS; ++x) ssum[x] = 0;
+  for (int x = 0; x < FS; ++x)
+#pragma unroll
+    for (int pl = 0; pl < PS; ++pl) psum[x][pl] = 0;
 
   uint32_t rotA[PA], rotB[PB];
 #pragma unroll
@@ -187,132 +273,111 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
   for (int pl = 0; pl < PB; ++pl) rotB[pl] = (uint32_t)(4 * g - pl) & 31u;
 
+  // packed words of this lane's rows for one k-step
+  uint32_t wA[FA][PA], wB[FB][PB];
+  auto read_words = [&](const uint32_t *buf, int ks) {
+    const uint32_t *As = buf + (wa * FA * 32 + li) * LD + ks;
+    const uint32_t *Bs = buf + PA * TA * LD + (wb * FB * 32 + li) * LD + ks;
+#pragma unroll
+    for (int x = 0; x < FA; ++x)
+#pragma unroll
+      for (int pl = 0; pl < PA; ++pl) wA[x][pl] = As[(pl * TA + x * 32) * LD];
+#pragma unroll
+    for (int y = 0; y < FB; ++y)
+#pragma unroll
+      for (int pl = 0; pl < PB; ++pl) wB[y][pl] = Bs[(pl * TB + y * 32) * LD];
+  };
+  v4i af[FA], bf[FB];
+  auto expand_all = [&](v4i (&a)[FA], v4i (&b)[FB]) {
+#pragma unroll
+    for (int x = 0; x < FA; ++x) {
+      if (CONV) {
+#pragma unroll
+        for (int pl = 0; pl < PA; ++pl) psum[x][pl] += __popc(wA[x][pl]);
+      }
+      a[x] = expand_planes<PA>(wA[x], rotA);
+    }
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      if (!CONV) {
+#pragma unroll
+        for (int pl = 0; pl < PB; ++pl) psum[y][pl] += __popc(wB[y][pl]);
+      }
+      b[y] = expand_planes<PB>(wB[y], rotB);
+    }
+  };
+
+  // Software pipeline: while the matrix cores work on k-step s, the VALU expands the operands of
+  // k-step s+1 (also across the chunk boundary: the barrier that publishes chunk ch+1 sits before
+  // the last k-step of chunk ch).  Global loads run two chunks ahead, LDS holds two chunks.
+  constexpr int N_MFMA = FA * FB;
+  constexpr int N_VALU = FA * 8 * PA + FB * 8 * PB + FS * PS;
+  constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
+
   const int nchunks = (p.KW + KC - 1) / KC;
   fetch(0);
   stage(smem);
+  if (nchunks > 1) fetch(KC);
   __syncthreads();
+  read_words(smem, 0);
+  expand_all(af, bf);
   for (int ch = 0; ch < nchunks; ++ch) {
-    const uint32_t *buf = smem + (ch & 1) * BUF_WORDS;
-    const uint32_t *As = buf + (wa * FA * 32 + li) * LD;
-    const uint32_t *Bs = buf + PA * TA * LD + (wb * FB * 32 + li) * LD;
-    if (ch + 1 < nchunks) fetch((ch + 1) * KC);
+    const uint32_t *cur = smem + (ch & 1) * BUF_WORDS;
+    uint32_t *nxt = smem + ((ch + 1) & 1) * BUF_WORDS;
+    const bool more = ch + 1 < nchunks;
+    if (more) {
+      stage(nxt);  // every wave left this buffer before the barrier of the previous chunk
+      if (ch + 2 < nchunks) fetch((ch + 2) * KC);
+    }
 #pragma unroll
     for (int ks = 0; ks < KC; ++ks) {
-      v4i af[FA], bf[FB];
-#pragma unroll
-      for (int x = 0; x < FA; ++x) {
-        uint32_t w[PA];
-#pragma unroll
-        for (int pl = 0; pl < PA; ++pl) w[pl] = As[(pl * TA + x * 32) * LD + ks];
-        if (CONV && p.sym) {
-#pragma unroll
-          for (int pl = 0; pl < PA; ++pl) ssum[x] += __popc(w[pl]) << pl;
-        }
-        af[x] = expand_planes<PA>(w, rotA);
-      }
-#pragma unroll
-      for (int y = 0; y < FB; ++y) {
-        uint32_t w[PB];
-#pragma unroll
-        for (int pl = 0; pl < PB; ++pl) w[pl] = Bs[(pl * TB + y * 32) * LD + ks];
-        if (!CONV && p.sym) {
-#pragma unroll
-          for (int pl = 0; pl < PB; ++pl) ssum[y] += __popc(w[pl]) << pl;
-        }
-        bf[y] = expand_planes<PB>(w, rotB);
+      const bool last = ks == KC - 1;
+      if (last) __syncthreads();
+      v4i an[FA], bn[FB];
+      if (!last) {
+        read_words(cur, ks + 1);
+      } else if (more) {
+        read_words(nxt, 0);
       }
 #pragma unroll
       for (int x = 0; x < FA; ++x)
 #pragma unroll
         for (int y = 0; y < FB; ++y)
           acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[x], bf[y], acc[x][y], 0, 0, 0);
+      if (!last || more) {
+        expand_all(an, bn);
+#pragma unroll
+        for (int x = 0; x < FA; ++x) af[x] = an[x];
+#pragma unroll
+        for (int y = 0; y < FB; ++y) bf[y] = bn[y];
+#pragma unroll
+        for (int i = 0; i < N_MFMA; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);  // then its share of VALU work
+        }
+      }
     }
-    if (ch + 1 < nchunks) stage(smem + ((ch + 1) & 1) * BUF_WORDS);
-    __syncthreads();
   }
-  (void)PS;
+  int ssum[FS];
+#pragma unroll
+  for (int x = 0; x < FS; ++x) {
+    int t = 0;
+#pragma unroll
+    for (int pl = 0; pl < PS; ++pl) t += psum[x][pl] << pl;
+    ssum[x] = t;
+  }
 
   // ---- epilogue from registers ---------------------------------------------------------------
-  // accumulator register r of a block: row 8*(r/4) + 4*g + (r%4), column li
-  const bool packed = p.epi != APNN_EPI_INT32;
-  const bool pooled = p.pool != APNN_POOL_NONE;
-  const int w32 = p.rowsB >> 5;
-  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
-#pragma unroll
-  for (int x = 0; x < FA; ++x) {
-#pragma unroll
-    for (int y = 0; y < FB; ++y) {
+  // Every accumulator index below is a compile-time constant (static_for), so the accumulators
+  // stay in registers for the whole kernel.
+  static_for<0, FA>([&](auto xc) {
+    static_for<0, FB>([&](auto yc) {
+      constexpr int x = decltype(xc)::value, y = decltype(yc)::value;
       const int gcol = b0 + (wb * FB + y) * 32 + li;
       const int rbase = a0 + (wa * FA + x) * 32;
-      const bool col_ok = gcol < p.rowsB;
-      int v[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int rin = 8 * (r >> 2) + 4 * g + (r & 3);
-        int t = acc[x][y][r];
-        if (p.sym) {
-          int s;
-          if (CONV) {
-            s = __shfl(ssum[x], rin, 64);  // lane `rin` (< 32) holds the sum of row rin of block x
-          } else {
-            s = ssum[y];
-          }
-          t = 2 * t - p.wmax * s;
-        }
-        v[r] = t;
-      }
-      if (!packed) {
-        int *out = reinterpret_cast<int *>(p.out);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (col_ok && grow < p.rowsA) out[(long long)grow * p.rowsB + gcol] = v[r];
-        }
-      } else if (!pooled) {
-        uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
-          const bool ok = col_ok && grow < p.rowsA;
-          int code = 0;
-          if (ok) {
-            int t = v[r];
-            const long long o = (long long)grow * p.rowsB + gcol;
-            if (p.resid != nullptr) t += p.resid[o];
-            if (p.save_acc != nullptr) p.save_acc[o] = t;
-            code = quantize_code(p, t, gcol);
-          }
-          for (int b = 0; b < p.out_bits; ++b) {
-            const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
-            const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
-            if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
-          }
-        }
-      } else {
-        uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int grow = (rbase + 8 * q + 4 * g) >> 2;  // window index
-          const bool ok = col_ok && grow < out_rows_total;
-          int code = 0;
-          if (ok) {
-            if (p.pool == APNN_POOL_AVG2X2) {
-              code = quantize_code(p, (v[4 * q] + v[4 * q + 1] + v[4 * q + 2] + v[4 * q + 3]) / 4, gcol);
-            } else {
-              const int c0 = quantize_code(p, v[4 * q], gcol), c1 = quantize_code(p, v[4 * q + 1], gcol);
-              const int c2 = quantize_code(p, v[4 * q + 2], gcol), c3 = quantize_code(p, v[4 * q + 3], gcol);
-              code = max(max(c0, c1), max(c2, c3));
-            }
-          }
-          for (int b = 0; b < p.out_bits; ++b) {
-            const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
-            const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
-            if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
-          }
-        }
-      }
-    }
-  }
+      mfma_epilogue_block<CONV>(p, acc[x][y], ssum[CONV ? x : y], rbase, gcol, g, li);
+    });
+  });
 }
 
 template <int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV>
