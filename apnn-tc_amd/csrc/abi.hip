@@ -89,19 +89,19 @@ void fill_epilogue(KParams &p, const apnn_epilogue &e, void *out, long long out_
 
 typedef hipError_t (*valu_fn)(int, int, const KParams &, hipStream_t);
 
-valu_fn mfma_gemm_fn(int wb, int xb) {
-  if (wb == 1 && xb == 2) return apnn::mfma_gemm_1_2_x;
-  if (wb == 1 && xb == 3) return apnn::mfma_gemm_1_3_x;
-  if (wb == 1 && xb == 4) return apnn::mfma_gemm_1_4_x;
-  if (wb == 2 && xb == 2) return apnn::mfma_gemm_2_2_x;
+valu_fn mfma_gemm_fn(int wb, int xb, bool i8) {
+  if (wb == 1 && xb == 2) return i8 ? apnn::mfma_gemm_1_2_x : apnn::mfma4_gemm_1_2_x;
+  if (wb == 1 && xb == 3) return i8 ? apnn::mfma_gemm_1_3_x : apnn::mfma4_gemm_1_3_x;
+  if (wb == 1 && xb == 4) return i8 ? apnn::mfma_gemm_1_4_x : apnn::mfma4_gemm_1_4_x;
+  if (wb == 2 && xb == 2) return i8 ? apnn::mfma_gemm_2_2_x : apnn::mfma4_gemm_2_2_x;
   return nullptr;
 }
 
-valu_fn mfma_conv_fn(int xb, int wb) {
-  if (xb == 2 && wb == 1) return apnn::mfma_conv_2_1_x;
-  if (xb == 3 && wb == 1) return apnn::mfma_conv_3_1_x;
-  if (xb == 4 && wb == 1) return apnn::mfma_conv_4_1_x;
-  if (xb == 2 && wb == 2) return apnn::mfma_conv_2_2_x;
+valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
+  if (xb == 2 && wb == 1) return i8 ? apnn::mfma_conv_2_1_x : apnn::mfma4_conv_2_1_x;
+  if (xb == 3 && wb == 1) return i8 ? apnn::mfma_conv_3_1_x : apnn::mfma4_conv_3_1_x;
+  if (xb == 4 && wb == 1) return i8 ? apnn::mfma_conv_4_1_x : apnn::mfma4_conv_4_1_x;
+  if (xb == 2 && wb == 2) return i8 ? apnn::mfma_conv_2_2_x : apnn::mfma4_conv_2_2_x;
   return nullptr;
 }
 
@@ -160,7 +160,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
-  if ((d->path >> 16) != 0 || (path != APNN_PATH_AUTO && path != APNN_PATH_VALU && path != APNN_PATH_MFMA))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_I8))
     return APNN_EINVAL;
   if ((rc = check_epilogue(d->epi, d->N, false, 0, 0))) return rc;
 
@@ -177,8 +177,8 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->D, d->M);
 
   int tile;
-  if (path == APNN_PATH_MFMA || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
-    valu_fn fn = mfma_gemm_fn(d->wb, d->xb);
+  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+    valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
     if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
     return (int)fn(4, tile, p, stream);
@@ -199,7 +199,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
-  if ((d->path >> 16) != 0 || (path != APNN_PATH_AUTO && path != APNN_PATH_VALU && path != APNN_PATH_MFMA))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_I8))
     return APNN_EINVAL;
   if (d->H + 2 * d->pad < d->R || d->Wd + 2 * d->pad < d->S) return APNN_EINVAL;
   const int Ho = (d->H + 2 * d->pad - d->R) / d->stride + 1;
@@ -236,8 +236,8 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
 
   int tile;
-  if (path == APNN_PATH_MFMA || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
-    valu_fn fn = mfma_conv_fn(d->xb, d->wb);
+  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+    valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
     if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
     return (int)fn(vw, tile, p, stream);

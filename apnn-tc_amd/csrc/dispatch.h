@@ -20,6 +20,8 @@ APNN_DECL_VALU(conv, 2, 2)
 
 #define APNN_DECL_MFMA(kind, pa, pb) \
   hipError_t mfma_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);
+#define APNN_DECL_MFMA4(kind, pa, pb) \
+  hipError_t mfma4_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);
 APNN_DECL_MFMA(gemm, 1, 2)
 APNN_DECL_MFMA(gemm, 1, 3)
 APNN_DECL_MFMA(gemm, 1, 4)
@@ -28,7 +30,16 @@ APNN_DECL_MFMA(conv, 2, 1)
 APNN_DECL_MFMA(conv, 3, 1)
 APNN_DECL_MFMA(conv, 4, 1)
 APNN_DECL_MFMA(conv, 2, 2)
+APNN_DECL_MFMA4(gemm, 1, 2)
+APNN_DECL_MFMA4(gemm, 1, 3)
+APNN_DECL_MFMA4(gemm, 1, 4)
+APNN_DECL_MFMA4(gemm, 2, 2)
+APNN_DECL_MFMA4(conv, 2, 1)
+APNN_DECL_MFMA4(conv, 3, 1)
+APNN_DECL_MFMA4(conv, 4, 1)
+APNN_DECL_MFMA4(conv, 2, 2)
 #undef APNN_DECL_MFMA
+#undef APNN_DECL_MFMA4
 
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
 constexpr int kMfmaTileCount = 4;

@@ -1,7 +1,16 @@
-// MFMA path: bit-planes are expanded to int8 in registers and contracted with
-// v_mfma_i32_32x32x32_i8, so a k-step of 32 elements costs one matrix instruction per 32x32 output
-// block whatever the bit widths are:  sum_ij 2^(i+j) popc(x_i & w_j) == sum_k xval[k] * wval[k]
-// with xval = sum_i 2^i x_i[k] (0..15) and wval likewise -- exact in int8 x int8 -> int32.
+// MFMA path: bit-planes are expanded in registers to small matrix-core operands and contracted on
+// the matrix cores:  sum_ij 2^(i+j) popc(x_i & w_j) == sum_k xval[k] * wval[k]  with
+// xval = sum_i 2^i x_i[k] and wval likewise.  Two operand encodings (template parameter CORE):
+//
+//  CORE_I8  v_mfma_i32_32x32x32_i8: operand bytes hold xval / wval (0..15); one instruction per 32x32
+//           block and 32 k, exact in int8 x int8 -> int32.
+//  CORE_F4  v_mfma_f32_32x32x64_f8f6f4 with FP4 (e2m1) operands: the codes 0..3 of e2m1 are the values
+//           0, 0.5, 1, 1.5, i.e. a 2-bit digit v is the code v and means v/2.  Operands are split into
+//           2-bit digits (plane pairs); digit pair (da, db) is one instruction per 32x32 block and
+//           64 k -- at the same issue cost as the int8 instruction, so twice its rate -- with the
+//           weight 4^(da+db) applied by the instruction's E8M0 block scale.  Products are multiples
+//           of 1/4 and partial sums stay far below 2^22, so the fp32 accumulators are exact and the
+//           result is acc * 4.
 //
 // Work-group = 4 waves arranged WA x WB, each wave owning an (FA*32) x (FB*32) output tile
 // (FA*FB accumulator blocks of 16 registers).  The *packed* planes are staged through LDS
@@ -16,9 +25,9 @@
 // Symmetric (+-) weights use the closed form  2*raw - wmax * (activation row sum); the row sums
 // come from popcounts of the packed words the wave already holds.
 //
-// The epilogue works from the accumulator registers: a 32-lane half holds 32 consecutive channels
-// of one output row, so one ballot per output bit yields the two MSB-first words of two rows, and
-// the four rows of a 2x2 pooling window (pool order) are four consecutive accumulator registers.
+// The epilogue passes each wave's tile through an LDS slab, 32 rows at a time, to turn the
+// matrix-core register layout into row-major order: stores are contiguous, and 64 consecutive
+// channels sit in the 64 lanes so that one ballot per output bit yields two MSB-first words.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -31,7 +40,29 @@
 namespace apnn {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+enum { CORE_I8 = 0, CORE_F4 = 1 };
+
+// FP4 operand for digit D (planes 2D and, if present, 2D+1) of a P-plane row word: nibble c of
+// result word t is the digit of element 4c + t.
+template <int P, int D>
+__device__ __forceinline__ v8i expand_fp4(const uint32_t (&w)[P]) {
+  v8i out = {0, 0, 0, 0, 0, 0, 0, 0};
+  const uint32_t x0 = w[2 * D];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    uint32_t word = (x0 >> t) & 0x11111111u;
+    if constexpr (2 * D + 1 < P) {
+      const uint32_t x1 = w[2 * D + 1];
+      word |= (t == 0 ? (x1 << 1) : (x1 >> (t - 1))) & 0x22222222u;
+    }
+    out[t] = (int)word;
+  }
+  return out;
+}
 
 template <int P>
 __device__ __forceinline__ v4i expand_planes(const uint32_t (&w)[P], const uint32_t (&rot)[P]) {
@@ -57,81 +88,90 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// Output stage for one 32x32 accumulator block.  Register r of the block holds
-// row 8*(r/4) + 4*g + (r%4), column li (g = lane / 32, li = lane % 32).
-// ssum: activation sum of row li of this block (CONV) or of column li (GEMM entry points).
-template <bool CONV>
-__device__ __forceinline__ void mfma_epilogue_block(const KParams &p, const v16i &blk, int ssum, int rbase,
-                                                    int gcol, int g, int li) {
-  const bool col_ok = gcol < p.rowsB;
-  const int w32 = p.rowsB >> 5;
-  int v[16];
-  static_for<0, 16>([&](auto rc) {
-    constexpr int r = decltype(rc)::value;
-    int t = blk[r];
-    if (p.sym) {
-      const int rin = 8 * (r >> 2) + 4 * g + (r & 3);
-      const int s = CONV ? __shfl(ssum, rin, 64) : ssum;
-      t = 2 * t - p.wmax * s;
-    }
-    v[r] = t;
-  });
+// Output stage of one wave for a 32-row slab of its tile, staged in LDS as slab[32][NCOLS + 1]
+// (row-major, so the 64 lanes walk 64 consecutive output channels).  rowsum / colsum hold the
+// activation sums for the symmetric-weight correction (rows for convolution, columns for the GEMM
+// entry points).  Called by all 64 lanes of the wave; no other wave touches this slab.
+template <int NCOLS, bool CONV>
+__device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab, const int *rowsum,
+                                              const int *colsum, int rbase, int cbase, int lane) {
+  constexpr int LDT = NCOLS + 1;
+  auto value = [&](int row, int col) {
+    int v = slab[row * LDT + col];
+    if (p.sym) v = 2 * v - p.wmax * (CONV ? rowsum[row] : colsum[col]);
+    return v;
+  };
   if (p.epi == APNN_EPI_INT32) {
     int *out = reinterpret_cast<int *>(p.out);
-    static_for<0, 16>([&](auto rc) {
-      constexpr int r = decltype(rc)::value;
-      const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
-      if (col_ok && grow < p.rowsA) out[(long long)grow * p.rowsB + gcol] = v[r];
-    });
-  } else if (p.pool == APNN_POOL_NONE) {
-    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-    static_for<0, 16>([&](auto rc) {
-      constexpr int r = decltype(rc)::value;
-      const int grow = rbase + 8 * (r >> 2) + 4 * g + (r & 3);
-      const bool ok = col_ok && grow < p.rowsA;
-      int code = 0;
-      if (ok) {
-        int t = v[r];
-        const long long o = (long long)grow * p.rowsB + gcol;
-        if (p.resid != nullptr) t += p.resid[o];
-        if (p.save_acc != nullptr) p.save_acc[o] = t;
-        code = quantize_code(p, t, gcol);
-      }
-      for (int b = 0; b < p.out_bits; ++b) {
-        const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
-        const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
-        if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
-      }
-    });
-  } else {
-    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-    const int out_rows_total = p.rowsA / 4;
-    static_for<0, 4>([&](auto qc) {
-      constexpr int q = decltype(qc)::value;
-      const int grow = (rbase + 8 * q + 4 * g) >> 2;  // 2x2 window index
-      const bool ok = col_ok && grow < out_rows_total;
-      int code = 0;
-      if (ok) {
-        if (p.pool == APNN_POOL_AVG2X2) {
-          code = quantize_code(p, (v[4 * q] + v[4 * q + 1] + v[4 * q + 2] + v[4 * q + 3]) / 4, gcol);
-        } else {
-          const int c0 = quantize_code(p, v[4 * q], gcol), c1 = quantize_code(p, v[4 * q + 1], gcol);
-          const int c2 = quantize_code(p, v[4 * q + 2], gcol), c3 = quantize_code(p, v[4 * q + 3], gcol);
-          code = max(max(c0, c1), max(c2, c3));
+    if ((p.rowsB & 3) == 0) {
+      // 4 channels per lane: a wave writes 1 KiB of contiguous output per step
+      for (int e = lane * 4; e < 32 * NCOLS; e += 256) {
+        const int row = e / NCOLS, col = e % NCOLS;
+        const int grow = rbase + row, gcol = cbase + col;
+        if (grow < p.rowsA && gcol < p.rowsB) {
+          int4 v4;
+          v4.x = value(row, col);
+          v4.y = value(row, col + 1);
+          v4.z = value(row, col + 2);
+          v4.w = value(row, col + 3);
+          *reinterpret_cast<int4 *>(out + (long long)grow * p.rowsB + gcol) = v4;
         }
       }
-      for (int b = 0; b < p.out_bits; ++b) {
-        const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
-        const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
-        if (ok && li == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
+    } else {
+      for (int e = lane; e < 32 * NCOLS; e += 64) {
+        const int row = e / NCOLS, col = e % NCOLS;
+        const int grow = rbase + row, gcol = cbase + col;
+        if (grow < p.rowsA && gcol < p.rowsB) out[(long long)grow * p.rowsB + gcol] = value(row, col);
       }
-    });
+    }
+    return;
+  }
+  uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+  const int w32 = p.rowsB >> 5;
+  const bool pooled = p.pool != APNN_POOL_NONE;
+  const int n_out = pooled ? 8 : 32;
+  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
+  const int row_base = pooled ? rbase / 4 : rbase;
+  for (int e = lane; e < n_out * NCOLS; e += 64) {
+    const int orow = e / NCOLS, col = e % NCOLS;
+    const int grow = row_base + orow, gcol = cbase + col;
+    const bool ok = grow < out_rows_total && gcol < p.rowsB;
+    int code = 0;
+    if (ok) {
+      if (!pooled) {
+        int v = value(orow, col);
+        const long long o = (long long)grow * p.rowsB + gcol;
+        if (p.resid != nullptr) v += p.resid[o];
+        if (p.save_acc != nullptr) p.save_acc[o] = v;
+        code = quantize_code(p, v, gcol);
+      } else {
+        const int t0 = value(4 * orow, col), t1 = value(4 * orow + 1, col);
+        const int t2 = value(4 * orow + 2, col), t3 = value(4 * orow + 3, col);
+        if (p.pool == APNN_POOL_AVG2X2) {
+          code = quantize_code(p, (t0 + t1 + t2 + t3) / 4, gcol);
+        } else {
+          code = max(max(quantize_code(p, t0, gcol), quantize_code(p, t1, gcol)),
+                     max(quantize_code(p, t2, gcol), quantize_code(p, t3, gcol)));
+        }
+      }
+    }
+    for (int b = 0; b < p.out_bits; ++b) {
+      const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
+      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
+      if (ok && (lane & 31) == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
+    }
   }
 }
 
-template <int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV>
-__global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
+__global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   static_assert(WA * WB == 4, "four waves per work-group");
+  constexpr bool F4 = CORE == CORE_F4;
+  constexpr int WPS = F4 ? 2 : 1;                 // packed words per row consumed by one k-step
+  constexpr int DA = F4 ? (PA + 1) / 2 : 1;       // operand digits (FP4: plane pairs)
+  constexpr int DB = F4 ? (PB + 1) / 2 : 1;
+  using AccT = typename std::conditional<F4, v16f, v16i>::type;
+  using FragT = typename std::conditional<F4, v8i, v4i>::type;
   constexpr int NT = 256;
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
   constexpr int KC = 8;              // k-words (32 elements each) per staged chunk
@@ -249,7 +289,7 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
     }
   };
 
-  v16i acc[FA][FB];
+  AccT acc[FA][FB];
 #pragma unroll
   for (int x = 0; x < FA; ++x)
 #pragma unroll
@@ -276,8 +316,10 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
   // packed words of this lane's rows for one k-step
   uint32_t wA[FA][PA], wB[FB][PB];
   auto read_words = [&](const uint32_t *buf, int ks) {
-    const uint32_t *As = buf + (wa * FA * 32 + li) * LD + ks;
-    const uint32_t *Bs = buf + PA * TA * LD + (wb * FB * 32 + li) * LD + ks;
+    // CORE_F4: the two lane halves take the two words of the 64-element k-step
+    const int kw = ks * WPS + (F4 ? g : 0);
+    const uint32_t *As = buf + (wa * FA * 32 + li) * LD + kw;
+    const uint32_t *Bs = buf + PA * TA * LD + (wb * FB * 32 + li) * LD + kw;
 #pragma unroll
     for (int x = 0; x < FA; ++x)
 #pragma unroll
@@ -287,15 +329,19 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
       for (int pl = 0; pl < PB; ++pl) wB[y][pl] = Bs[(pl * TB + y * 32) * LD];
   };
-  v4i af[FA], bf[FB];
-  auto expand_all = [&](v4i (&a)[FA], v4i (&b)[FB]) {
+  FragT af[FA][DA], bf[FB][DB];
+  auto expand_all = [&](FragT (&a)[FA][DA], FragT (&b)[FB][DB]) {
 #pragma unroll
     for (int x = 0; x < FA; ++x) {
       if (CONV) {
 #pragma unroll
         for (int pl = 0; pl < PA; ++pl) psum[x][pl] += __popc(wA[x][pl]);
       }
-      a[x] = expand_planes<PA>(wA[x], rotA);
+      if constexpr (F4) {
+        static_for<0, DA>([&](auto dc) { a[x][decltype(dc)::value] = expand_fp4<PA, decltype(dc)::value>(wA[x]); });
+      } else {
+        a[x][0] = expand_planes<PA>(wA[x], rotA);
+      }
     }
 #pragma unroll
     for (int y = 0; y < FB; ++y) {
@@ -303,15 +349,44 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
         for (int pl = 0; pl < PB; ++pl) psum[y][pl] += __popc(wB[y][pl]);
       }
-      b[y] = expand_planes<PB>(wB[y], rotB);
+      if constexpr (F4) {
+        static_for<0, DB>([&](auto dc) { b[y][decltype(dc)::value] = expand_fp4<PB, decltype(dc)::value>(wB[y]); });
+      } else {
+        b[y][0] = expand_planes<PB>(wB[y], rotB);
+      }
     }
+  };
+  auto mfma_all = [&]() {
+#pragma unroll
+    for (int x = 0; x < FA; ++x)
+#pragma unroll
+      for (int y = 0; y < FB; ++y) {
+        if constexpr (F4) {
+          static_for<0, DA>([&](auto dac) {
+            static_for<0, DB>([&](auto dbc) {
+              constexpr int da = decltype(dac)::value, db = decltype(dbc)::value;
+              if constexpr (da + db == 0) {
+                acc[x][y] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[x][da], bf[y][db], acc[x][y], 4, 4,
+                                                                            0, 0, 0, 0);
+              } else {
+                // E8M0 block scales: 127 = 2^0 on A, 127 + 2*(da+db) = 4^(da+db) on B
+                acc[x][y] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    af[x][da], bf[y][db], acc[x][y], 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F + 0x02020202 * (da + db));
+              }
+            });
+          });
+        } else {
+          acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[x][0], bf[y][0], acc[x][y], 0, 0, 0);
+        }
+      }
   };
 
   // Software pipeline: while the matrix cores work on k-step s, the VALU expands the operands of
   // k-step s+1 (also across the chunk boundary: the barrier that publishes chunk ch+1 sits before
   // the last k-step of chunk ch).  Global loads run two chunks ahead, LDS holds two chunks.
-  constexpr int N_MFMA = FA * FB;
-  constexpr int N_VALU = FA * 8 * PA + FB * 8 * PB + FS * PS;
+  constexpr int NKS = KC / WPS;  // k-steps per chunk
+  constexpr int N_MFMA = FA * FB * DA * DB;
+  constexpr int N_VALU = (F4 ? 7 : 8) * (FA * PA + FB * PB) + FS * PS;
   constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
 
   const int nchunks = (p.KW + KC - 1) / KC;
@@ -329,34 +404,35 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
       stage(nxt);  // every wave left this buffer before the barrier of the previous chunk
       if (ch + 2 < nchunks) fetch((ch + 2) * KC);
     }
-#pragma unroll
-    for (int ks = 0; ks < KC; ++ks) {
-      const bool last = ks == KC - 1;
-      if (last) __syncthreads();
-      v4i an[FA], bn[FB];
-      if (!last) {
-        read_words(cur, ks + 1);
-      } else if (more) {
-        read_words(nxt, 0);
-      }
+    auto advance = [&]() {
+      FragT an[FA][DA], bn[FB][DB];
+      expand_all(an, bn);
 #pragma unroll
       for (int x = 0; x < FA; ++x)
 #pragma unroll
-        for (int y = 0; y < FB; ++y)
-          acc[x][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[x], bf[y], acc[x][y], 0, 0, 0);
-      if (!last || more) {
-        expand_all(an, bn);
+        for (int d = 0; d < DA; ++d) af[x][d] = an[x][d];
 #pragma unroll
-        for (int x = 0; x < FA; ++x) af[x] = an[x];
+      for (int y = 0; y < FB; ++y)
 #pragma unroll
-        for (int y = 0; y < FB; ++y) bf[y] = bn[y];
+        for (int d = 0; d < DB; ++d) bf[y][d] = bn[y][d];
 #pragma unroll
-        for (int i = 0; i < N_MFMA; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);  // then its share of VALU work
-        }
+      for (int i = 0; i < N_MFMA; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);  // then its share of VALU work
       }
+    };
+    // k-steps 0 .. NKS-2 (kept as a real loop: one scheduling region per k-step)
+#pragma unroll 1
+    for (int ks = 0; ks + 1 < NKS; ++ks) {
+      read_words(cur, ks + 1);
+      mfma_all();
+      advance();
     }
+    // last k-step of the chunk: publish the next chunk first, then prefetch its first operands
+    __syncthreads();
+    if (more) read_words(nxt, 0);
+    mfma_all();
+    if (more) advance();
   }
   int ssum[FS];
 #pragma unroll
@@ -364,29 +440,55 @@ __global__ __launch_bounds__(256) void apnn_mfma_kernel(const KParams p) {
     int t = 0;
 #pragma unroll
     for (int pl = 0; pl < PS; ++pl) t += psum[x][pl] << pl;
+    if (F4) t += __shfl_xor(t, 32, 64);  // the lane halves counted different words of the row
     ssum[x] = t;
   }
 
-  // ---- epilogue from registers ---------------------------------------------------------------
-  // Every accumulator index below is a compile-time constant (static_for), so the accumulators
-  // stay in registers for the whole kernel.
+  // ---- epilogue: one 32-row slab of the wave tile at a time through LDS ----------------------
+  // Accumulator indices are compile-time constants (static_for) so they stay in registers; the
+  // slab turns the matrix-core layout (register r of a block = row 8*(r/4) + 4*g + r%4, column li)
+  // into row-major order for coalesced stores and 64-channel ballots.
+  constexpr int NCOLS = FB * 32, LDT = NCOLS + 1;
+  constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS;
+  __syncthreads();  // every wave is done with the staging buffers
+  int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
+  int *rowsum = slab + 32 * LDT;
+  int *colsum = rowsum + 32;
+  if (!CONV && g == 0) {
+#pragma unroll
+    for (int y = 0; y < FB; ++y) colsum[y * 32 + li] = ssum[CONV ? 0 : y];
+  }
   static_for<0, FA>([&](auto xc) {
+    constexpr int x = decltype(xc)::value;
+    if (CONV && g == 0) rowsum[li] = ssum[CONV ? x : 0];
     static_for<0, FB>([&](auto yc) {
-      constexpr int x = decltype(xc)::value, y = decltype(yc)::value;
-      const int gcol = b0 + (wb * FB + y) * 32 + li;
-      const int rbase = a0 + (wa * FA + x) * 32;
-      mfma_epilogue_block<CONV>(p, acc[x][y], ssum[CONV ? x : y], rbase, gcol, g, li);
+      constexpr int y = decltype(yc)::value;
+      static_for<0, 16>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        int v;
+        if constexpr (F4) {
+          v = __float2int_rn(acc[x][y][r] * 4.0f);
+        } else {
+          v = acc[x][y][r];
+        }
+        slab[(8 * (r >> 2) + 4 * g + (r & 3)) * LDT + y * 32 + li] = v;
+      });
     });
+    // LDS operations of one wave complete in order: the reads below see the writes above, and the
+    // next slab's writes come after these reads
+    wave_epilogue<NCOLS, CONV>(p, slab, rowsum, colsum, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane);
   });
 }
 
-template <int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV>
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
   constexpr int LD = 9;
-  constexpr size_t smem_bytes = 2ull * (PA * TA + PB * TB) * LD * sizeof(uint32_t);
-  static_assert(smem_bytes <= 160 * 1024, "LDS budget of a gfx950 work-group");
-  auto kern = apnn_mfma_kernel<PA, PB, FA, FB, WA, WB, VW, CONV>;
+  constexpr size_t stage_bytes = 2ull * (PA * TA + PB * TB) * LD * sizeof(uint32_t);
+  constexpr size_t slab_bytes = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32) * sizeof(int);
+  constexpr size_t smem_bytes = stage_bytes > slab_bytes ? stage_bytes : slab_bytes;
+  static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
+  auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>;
   if (smem_bytes > 64 * 1024) {
     static bool raised = false;  // per instantiation; a repeated call is harmless
     if (!raised) {
@@ -403,13 +505,13 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
 
 enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_COUNT = 4 };
 
-template <int PA, int PB, int VW, bool CONV>
+template <int CORE, int PA, int PB, int VW, bool CONV>
 inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t stream) {
   switch (tile) {
-    case MT_256x256: return launch_mfma<PA, PB, 4, 4, 2, 2, VW, CONV>(p, stream);
-    case MT_128x128: return launch_mfma<PA, PB, 2, 2, 2, 2, VW, CONV>(p, stream);
-    case MT_128x64: return launch_mfma<PA, PB, 1, 2, 4, 1, VW, CONV>(p, stream);
-    default: return launch_mfma<PA, PB, 1, 1, 2, 2, VW, CONV>(p, stream);
+    case MT_256x256: return launch_mfma<CORE, PA, PB, 4, 4, 2, 2, VW, CONV, 1>(p, stream);
+    case MT_128x128: return launch_mfma<CORE, PA, PB, 2, 2, 2, 2, VW, CONV, 2>(p, stream);
+    case MT_128x64: return launch_mfma<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 2>(p, stream);
+    default: return launch_mfma<CORE, PA, PB, 1, 1, 2, 2, VW, CONV, 2>(p, stream);
   }
 }
 

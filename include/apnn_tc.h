@@ -87,7 +87,10 @@ enum { APNN_EPI_INT32 = 0,    /* int32 result                                   
 enum { APNN_POOL_NONE = 0,
        APNN_POOL_AVG2X2 = 1,  /* (v0+v1+v2+v3)/4 on the int32 result before quantizing (LIB/68:280-292) */
        APNN_POOL_MAX2X2 = 2 };/* max over the 2x2 window of the quantized codes                     */
-enum { APNN_PATH_AUTO = 0, APNN_PATH_VALU = 1, APNN_PATH_MFMA = 2 };
+enum { APNN_PATH_AUTO = 0,
+       APNN_PATH_VALU = 1,     /* v_and + v_bcnt popcount on packed words                           */
+       APNN_PATH_MFMA = 2,     /* planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4      */
+       APNN_PATH_MFMA_I8 = 3 };/* planes expanded to int8 operands of v_mfma_i32_32x32x32_i8         */
 /* `path` fields: low byte = APNN_PATH_*; bits 8..15 = 0 (library picks the tile shape) or
  * 1 + tile index to pin it (tuning / test coverage of every tile shape; APNN_EINVAL if the
  * chosen kernel family has no such tile or the epilogue cannot use it). */

@@ -50,7 +50,7 @@ def test_gemm_named_entry_golden(G, wb, xb):
     assert np.array_equal(gotp, O.lowbits_pack(_golden()["gemm_" + name], M, N, xb))
 
 
-PATHS = [1, 2]   # APNN_PATH_VALU, APNN_PATH_MFMA
+PATHS = [1, 2, 3]   # APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8
 
 
 @pytest.mark.parametrize("path", PATHS)
@@ -102,7 +102,7 @@ def test_gemm_symmetric_weights(G, wb, xb, path):
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=1))
 
 
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3)])
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (3, 0), (3, 1), (3, 2), (3, 3)])
 def test_gemm_bn_epilogue_with_residual(G, tile, path):
     rng = np.random.default_rng(91 + tile)
     M, N, K, wb, xb, ob = 48, 160, 256, 1, 2, 2
@@ -201,7 +201,7 @@ def test_conv_every_tile(G, tile, path):
 
 
 @pytest.mark.parametrize("pool", [0, 1, 2])
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3)])
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (3, 0), (3, 1), (3, 2), (3, 3)])
 def test_conv_bn_epilogue(G, pool, tile, path):
     """BN-threshold requantize to a bits (+ residual / saved accumulator when not pooling,
     + avg / max pooling), packed for the next layer."""
