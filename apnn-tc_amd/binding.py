@@ -25,7 +25,8 @@ _ci = ctypes.c_int
 
 class Epilogue(ctypes.Structure):
     _fields_ = [("mode", _ci), ("out_bits", _ci), ("pool", _ci),
-                ("thresholds", _vp), ("flip", _vp), ("residual", _vp), ("save_acc", _vp)]
+                ("thresholds", _vp), ("flip", _vp), ("residual", _vp), ("save_acc", _vp),
+                ("residual_planes", _vp), ("residual_bits", _ci), ("residual_scale", _ci)]
 
 
 class GemmDesc(ctypes.Structure):
@@ -48,7 +49,8 @@ _GEMM_NAMES = ["apmm_w1a2", "apmm_w1a3", "apmm_w1a4", "apmm_w2a2",
 _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2",
                "APConv_w1a2_pack", "APConv_w1a3_pack", "APConv_w1a4_pack", "APConv_w2a2_pack",
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
-DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits",
+DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
+                                                "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
                                                 "apnn_device_cus", "apnn_version"]
 
 
@@ -100,6 +102,14 @@ def lib():
         L.apnn_conv.restype = _ci
         L.apnn_pack_bits.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]
         L.apnn_pack_bits.restype = _ci
+        L.apnn_conv_i8_bn.argtypes = [_vp] * 5 + [_ci] * 10 + [_vp]
+        L.apnn_conv_i8_bn.restype = _ci
+        L.apnn_pool_pack.argtypes = [_vp, _vp] + [_ci] * 9 + [_vp]
+        L.apnn_pool_pack.restype = _ci
+        L.apnn_unpack_sum.argtypes = [_vp, _vp, ctypes.c_longlong] + [_ci] * 5 + [_vp]
+        L.apnn_unpack_sum.restype = _ci
+        L.apnn_fc_i8.argtypes = [_vp] * 6 + [_ci] * 3 + [_vp]
+        L.apnn_fc_i8.restype = _ci
         L.apnn_device_cus.argtypes = []
         L.apnn_device_cus.restype = _ci
         L.apnn_version.argtypes = []

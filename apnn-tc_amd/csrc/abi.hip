@@ -62,15 +62,20 @@ int check_epilogue(const apnn_epilogue &e, int rowsB, bool is_conv, int Ho, int 
   if (e.mode != APNN_EPI_INT32 && e.mode != APNN_EPI_LOWBITS && e.mode != APNN_EPI_BN) return APNN_EINVAL;
   if (e.pool != APNN_POOL_NONE && e.pool != APNN_POOL_AVG2X2 && e.pool != APNN_POOL_MAX2X2) return APNN_EINVAL;
   if (e.mode == APNN_EPI_INT32) {
-    if (e.pool != APNN_POOL_NONE || e.residual != nullptr || e.save_acc != nullptr) return APNN_EINVAL;
+    if (e.pool != APNN_POOL_NONE || e.residual != nullptr || e.save_acc != nullptr || e.residual_planes != nullptr)
+      return APNN_EINVAL;
     return APNN_OK;
+  }
+  if (e.residual_planes != nullptr) {
+    if (e.residual_bits < 1 || e.residual_bits > 8) return APNN_EINVAL;
+    if ((reinterpret_cast<uintptr_t>(e.residual_planes) & 3u) != 0) return APNN_EALIGN;
   }
   if (e.out_bits < 1 || e.out_bits > 8) return APNN_EINVAL;
   if (rowsB % 32 != 0) return APNN_EINVAL;
   if (e.mode == APNN_EPI_BN && e.thresholds == nullptr) return APNN_ENULL;
   if (e.pool != APNN_POOL_NONE) {
     if (!is_conv || (Ho & 1) || (Wo & 1)) return APNN_EINVAL;
-    if (e.residual != nullptr || e.save_acc != nullptr) return APNN_EINVAL;
+    if (e.residual != nullptr || e.save_acc != nullptr || e.residual_planes != nullptr) return APNN_EINVAL;
   }
   return APNN_OK;
 }
@@ -83,6 +88,9 @@ void fill_epilogue(KParams &p, const apnn_epilogue &e, void *out, long long out_
   p.flip = e.flip;
   p.resid = e.residual;
   p.save_acc = e.save_acc;
+  p.resid_planes = e.residual_planes;
+  p.resid_bits = e.residual_bits;
+  p.resid_scale = e.residual_scale;
   p.out = out;
   p.out_plane = out_rows * (p.rowsB / 32);
 }
@@ -337,6 +345,45 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
   if (values == nullptr || planes == nullptr) return APNN_ENULL;
   if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 32) return APNN_EINVAL;
   return (int)apnn::launch_pack_bits(values, planes, rows, C, cpad, bits, static_cast<hipStream_t>(s));
+}
+
+int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint8_t *codes, int32_t *acc_out,
+                    int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
+                    apnn_stream_t s) {
+  if (X == nullptr || Wt == nullptr || (codes == nullptr && acc_out == nullptr)) return APNN_ENULL;
+  if (codes != nullptr && thresholds == nullptr) return APNN_ENULL;
+  if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || COUT <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0)
+    return APNN_EINVAL;
+  if (H + 2 * pad < R || W + 2 * pad < S) return APNN_EINVAL;
+  if (codes != nullptr && (bits < 1 || bits > 8)) return APNN_EINVAL;
+  if ((long long)64 * R * S * C > 64 * 1024) return APNN_EUNSUPPORTED;  // filter block must fit in LDS
+  return (int)apnn::launch_conv_i8_bn(X, Wt, thresholds, codes, acc_out, B, H, W, C, COUT, R, S, stride, pad, bits,
+                                      static_cast<hipStream_t>(s));
+}
+
+int apnn_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits, int win,
+                   int stride, int pad, apnn_stream_t s) {
+  if (codes == nullptr || planes == nullptr) return APNN_ENULL;
+  if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 8) return APNN_EINVAL;
+  if (win <= 0 || stride <= 0 || pad < 0 || pad >= win || H + 2 * pad < win || W + 2 * pad < win) return APNN_EINVAL;
+  return (int)apnn::launch_pool_pack(codes, planes, B, H, W, C, cpad, bits, win, stride, pad,
+                                     static_cast<hipStream_t>(s));
+}
+
+int apnn_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad, int bits,
+                    int shift, apnn_stream_t s) {
+  if (planes == nullptr || out == nullptr) return APNN_ENULL;
+  if (rows_out <= 0 || group <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 8 || shift < 0 ||
+      shift > 16)
+    return APNN_EINVAL;
+  return (int)apnn::launch_unpack_sum(planes, out, rows_out, group, C, cpad, bits, shift, static_cast<hipStream_t>(s));
+}
+
+int apnn_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
+               int32_t *acc_out, int B, int N, int K, apnn_stream_t s) {
+  if (X == nullptr || Wt == nullptr || scale == nullptr || bias == nullptr || out == nullptr) return APNN_ENULL;
+  if (B <= 0 || N <= 0 || K <= 0) return APNN_EINVAL;
+  return (int)apnn::launch_fc_i8(X, Wt, scale, bias, out, acc_out, B, N, K, static_cast<hipStream_t>(s));
 }
 
 int apnn_device_cus(void) { return device_cus(); }

@@ -22,6 +22,17 @@ __device__ __forceinline__ int quantize_code(const KParams &p, int v, int gcol) 
   return code;
 }
 
+// shortcut contribution of a packed residual branch for output element (grow, gcol)
+__device__ __forceinline__ int packed_residual(const KParams &p, int grow, int gcol) {
+  const int w32 = p.rowsB >> 5;
+  const long long plane = (long long)p.rowsA * w32;
+  const long long wi = (long long)grow * w32 + (gcol >> 5);
+  const int sh = 31 - (gcol & 31);
+  int code = 0;
+  for (int b = 0; b < p.resid_bits; ++b) code |= (int)((p.resid_planes[b * plane + wi] >> sh) & 1u) << b;
+  return code * p.resid_scale;
+}
+
 // tile: LDS, [TA][TB + 1] int32, row r of the tile is output row a0 + r (or, in pool order, rows
 // 4i..4i+3 are the 2x2 window a0/4 + i).  Must be called by every thread of the block after a
 // __syncthreads() that made the tile visible.
@@ -52,6 +63,7 @@ __device__ __forceinline__ void epilogue_packed(const KParams &p, const int *til
         int v = tile[orow * LDT + col];
         const long long o = (long long)grow * p.rowsB + gcol;
         if (p.resid != nullptr) v += p.resid[o];
+        if (p.resid_planes != nullptr) v += packed_residual(p, grow, gcol);
         if (p.save_acc != nullptr) p.save_acc[o] = v;
         code = quantize_code(p, v, gcol);
       } else {

@@ -38,6 +38,8 @@ struct KParams {
   const uint8_t *flip;
   const int32_t *resid;
   int32_t *save_acc;
+  const uint32_t *resid_planes;  // packed shortcut codes [resid_bits][rows][rowsB/32]
+  int resid_bits, resid_scale;
   void *out;
   long long out_plane;       // packed output: plane stride in words
 };

@@ -142,6 +142,7 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
         int v = value(orow, col);
         const long long o = (long long)grow * p.rowsB + gcol;
         if (p.resid != nullptr) v += p.resid[o];
+        if (p.resid_planes != nullptr) v += packed_residual(p, grow, gcol);
         if (p.save_acc != nullptr) p.save_acc[o] = v;
         code = quantize_code(p, v, gcol);
       } else {

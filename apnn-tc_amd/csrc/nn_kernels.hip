@@ -1,0 +1,192 @@
+// Kernels on either side of the low-bit path of a network: the int8 first convolution with its
+// threshold quantizer, max-pool + bit-plane packing of the resulting codes, global average pooling
+// of packed codes, code unpacking and the int8 classifier.
+#include <hip/hip_runtime.h>
+
+#include "../../include/apnn_tc.h"
+#include "dispatch.h"
+
+namespace apnn {
+
+// ---- int8 first convolution + per-channel thresholds -> codes ------------------------------------
+// X: [B][H][W][C] int8, Wt: [COUT][R][S][C] int8 (C tiny: 3), thr: [COUT][2^bits-1] int32.
+// One work-group computes a strip of 64 output pixels x COUT_T=64 channels; the filter block is
+// staged in LDS once, each thread owns one pixel and 16 channels.
+template <int COUT_T>
+__global__ __launch_bounds__(256) void conv_i8_bn_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                         const int32_t *__restrict__ thr,
+                                                         uint8_t *__restrict__ codes, int32_t *__restrict__ acc_out,
+                                                         int B, int H, int W, int C, int COUT, int R, int S,
+                                                         int stride, int pad, int Ho, int Wo, int bits) {
+  extern __shared__ int8_t wlds[];  // [COUT_T][R*S*C]
+  const int K = R * S * C;
+  const int co0 = blockIdx.y * COUT_T;
+  for (int i = threadIdx.x; i < COUT_T * K; i += 256) {
+    const int co = co0 + i / K;
+    wlds[i] = co < COUT ? Wt[(long long)co * K + (i % K)] : (int8_t)0;
+  }
+  __syncthreads();
+  const int pl = threadIdx.x & 63;          // pixel within the strip
+  const int cg = threadIdx.x >> 6;          // channel group: 16 channels
+  const long long pix = (long long)blockIdx.x * 64 + pl;
+  const long long npix = (long long)B * Ho * Wo;
+  if (pix >= npix) return;
+  const int ox = (int)(pix % Wo);
+  const int oy = (int)((pix / Wo) % Ho);
+  const int b = (int)(pix / ((long long)Wo * Ho));
+  int acc[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) acc[j] = 0;
+  for (int r = 0; r < R; ++r) {
+    const int iy = oy * stride + r - pad;
+    if (iy < 0 || iy >= H) continue;
+    for (int s = 0; s < S; ++s) {
+      const int ix = ox * stride + s - pad;
+      if (ix < 0 || ix >= W) continue;
+      const int8_t *xp = X + (((long long)b * H + iy) * W + ix) * C;
+      const int8_t *wp = wlds + (cg * 16) * K + (r * S + s) * C;
+      for (int c = 0; c < C; ++c) {
+        const int xv = xp[c];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] += xv * (int)wp[j * K + c];
+      }
+    }
+  }
+  const int nt = (1 << bits) - 1;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int co = co0 + cg * 16 + j;
+    if (co >= COUT) break;
+    if (acc_out != nullptr) acc_out[pix * COUT + co] = acc[j];
+    if (codes != nullptr) {
+      int code = 0;
+      for (int k = 0; k < nt; ++k) code += acc[j] >= thr[co * nt + k] ? 1 : 0;
+      codes[pix * COUT + co] = (uint8_t)code;
+    }
+  }
+}
+
+// ---- max-pool on codes + bit-plane packing ---------------------------------------------------------
+// codes: [B][H][W][C] uint8 -> planes [bits][B*Ho*Wo][cpad/32], window win x win, stride, pad
+// (out-of-image taps ignored).  One wave per (pixel, 64-channel group).
+__global__ __launch_bounds__(256) void pool_pack_kernel(const uint8_t *__restrict__ codes, uint32_t *__restrict__ planes,
+                                                        int B, int H, int W, int C, int cpad, int bits, int win,
+                                                        int stride, int pad, int Ho, int Wo) {
+  const int lane = threadIdx.x & 63;
+  const int cw = cpad >> 5;
+  const int groups = (cpad + 63) >> 6;
+  const long long rows = (long long)B * Ho * Wo;
+  const long long total = rows * groups;
+  for (long long gidx = (long long)blockIdx.x * 4 + (threadIdx.x >> 6); gidx < total; gidx += (long long)gridDim.x * 4) {
+    const long long row = gidx / groups;
+    const int c = (int)(gidx % groups) * 64 + lane;
+    const int ox = (int)(row % Wo), oy = (int)((row / Wo) % Ho), b = (int)(row / ((long long)Wo * Ho));
+    int v = 0;
+    if (c < C) {
+      for (int r = 0; r < win; ++r) {
+        const int iy = oy * stride + r - pad;
+        if (iy < 0 || iy >= H) continue;
+        for (int s = 0; s < win; ++s) {
+          const int ix = ox * stride + s - pad;
+          if (ix < 0 || ix >= W) continue;
+          v = max(v, (int)codes[(((long long)b * H + iy) * W + ix) * C + c]);
+        }
+      }
+    }
+    for (int bit = 0; bit < bits; ++bit) {
+      const unsigned long long mask = __ballot((v >> bit) & 1);
+      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
+      const int wi = c >> 5;
+      if ((lane & 31) == 0 && wi < cw) planes[bit * rows * cw + row * cw + wi] = word;
+    }
+  }
+}
+
+// ---- packed codes -> int8 values (optionally summed over `group` consecutive rows) ---------------
+// planes: [bits][rows][cpad/32];  out[r][c] = (sum_{j<group} code[r*group + j][c]) >> shift, int8.
+// group = 1, shift = 0: plain unpacking.  group = H*W: global pooling of a feature map.
+__global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restrict__ planes, int8_t *__restrict__ out,
+                                                         long long rows_out, int group, int C, int cpad, int bits,
+                                                         int shift) {
+  const int cw = cpad >> 5;
+  const long long rows_in = rows_out * group;
+  const long long total = rows_out * C;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (long long)gridDim.x * blockDim.x) {
+    const long long r = i / C;
+    const int c = (int)(i % C);
+    int sum = 0;
+    for (int j = 0; j < group; ++j) {
+      const long long rin = r * group + j;
+      int code = 0;
+      for (int b = 0; b < bits; ++b)
+        code |= (int)((planes[b * rows_in * cw + rin * cw + (c >> 5)] >> (31 - (c & 31))) & 1u) << b;
+      sum += code;
+    }
+    out[i] = (int8_t)min(127, sum >> shift);
+  }
+}
+
+// ---- int8 classifier: out[b][n] = scale[n] * sum_k X[b][k] * Wt[n][k] + bias[n] -----------------
+// One wave per output; K % 4 == 0 handled by 4-byte dot products, tail by bytes.
+__global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                    const float *__restrict__ scale, const float *__restrict__ bias,
+                                                    float *__restrict__ out, int32_t *__restrict__ acc_out, int Bn,
+                                                    int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const long long o = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (o >= (long long)Bn * N) return;
+  const int b = (int)(o / N), n = (int)(o % N);
+  const int8_t *x = X + (long long)b * K;
+  const int8_t *w = Wt + (long long)n * K;
+  int acc = 0;
+  for (int k = lane; k < K; k += 64) acc += (int)x[k] * (int)w[k];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0) {
+    if (acc_out != nullptr) acc_out[o] = acc;
+    out[o] = (float)acc * scale[n] + bias[n];
+  }
+}
+
+hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
+                             int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
+                             hipStream_t s) {
+  const int Ho = (H + 2 * pad - R) / stride + 1, Wo = (W + 2 * pad - S) / stride + 1;
+  const long long npix = (long long)B * Ho * Wo;
+  const size_t lds = (size_t)64 * R * S * C;
+  dim3 grid((unsigned)((npix + 63) / 64), (unsigned)((COUT + 63) / 64));
+  hipLaunchKernelGGL(conv_i8_bn_kernel<64>, grid, dim3(256), lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT, R,
+                     S, stride, pad, Ho, Wo, bits);
+  return hipGetLastError();
+}
+
+hipError_t launch_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits,
+                            int win, int stride, int pad, hipStream_t s) {
+  const int Ho = (H + 2 * pad - win) / stride + 1, Wo = (W + 2 * pad - win) / stride + 1;
+  const long long total = (long long)B * Ho * Wo * ((cpad + 63) / 64);
+  long long blocks = (total + 3) / 4;
+  if (blocks > 262144) blocks = 262144;
+  hipLaunchKernelGGL(pool_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, codes, planes, B, H, W, C, cpad, bits,
+                     win, stride, pad, Ho, Wo);
+  return hipGetLastError();
+}
+
+hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad,
+                             int bits, int shift, hipStream_t s) {
+  long long blocks = (rows_out * C + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(unpack_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, s, planes, out, rows_out, group, C, cpad,
+                     bits, shift);
+  return hipGetLastError();
+}
+
+hipError_t launch_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
+                        int32_t *acc_out, int Bn, int N, int K, hipStream_t s) {
+  const long long outs = (long long)Bn * N;
+  hipLaunchKernelGGL(fc_i8_kernel, dim3((unsigned)((outs + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out, acc_out,
+                     Bn, N, K);
+  return hipGetLastError();
+}
+
+}  // namespace apnn

@@ -101,6 +101,7 @@ enum { APNN_WEIGHT_UNSIGNED = 0,   /* planes are an unsigned integer u (the refe
 /* Output stage shared by GEMM and convolution.  "channel" is the fast output index
  * (N for GEMM, COUT for convolution).
  *   v = acc (after AVG pooling if requested) + (residual ? residual[row][channel] : 0)
+ *         + (residual_planes ? residual_scale * code(residual_planes)[row][channel] : 0)
  *   save_acc (optional) receives v as int32 [rows][channels]   (cf. save_residual, NN/kernel.cuh:779-831)
  *   LOWBITS: code = v & (2^out_bits - 1)
  *   BN     : code = #{ k < 2^out_bits-1 : (flip[channel] ? -v : v) >= thresholds[channel][k] }
@@ -115,6 +116,10 @@ typedef struct apnn_epilogue {
   const uint8_t *flip;       /* device, [channels] or NULL (BN) */
   const int32_t *residual;   /* device, [rows][channels] int32 or NULL */
   int32_t *save_acc;         /* device, [rows][channels] int32 or NULL */
+  const uint32_t *residual_planes; /* device, packed codes [residual_bits][rows][channels/32] of a
+                                      shortcut branch (identity: the block input), or NULL */
+  int residual_bits;         /* 1..8 */
+  int residual_scale;        /* integer factor that brings the shortcut codes to accumulator scale */
 } apnn_epilogue;
 
 /* out[m][n] over W:[wb][M][K/32] (slow index) and X:[xb][N][K/32] (fast index). */
@@ -152,6 +157,35 @@ int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s);
  * values:[rows][C] uint32 codes -> planes:[bits][rows][cpad/32], channel c at bit 31-c%32,
  * pad channels zero.  cpad % 32 == 0, cpad >= C. */
 int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits, apnn_stream_t s);
+
+/* ---- layers on either side of the low-bit path ------------------------------------------------ */
+
+/* int8 NHWC convolution with zero padding (the first layer of a network, cf. the int8 convention of
+ * cutlass_nn/src/config.h:215-255: int8 operands, int32 accumulate), followed by per-channel
+ * thresholds: code = #{k : acc >= thresholds[c][k]}.
+ * X:[B][H][W][C] int8, Wt:[COUT][R][S][C] int8; codes:[B][Ho][Wo][COUT] uint8 (NULL to skip),
+ * acc_out:[B][Ho][Wo][COUT] int32 (NULL to skip); thresholds may be NULL when codes is NULL. */
+int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint8_t *codes, int32_t *acc_out,
+                    int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
+                    apnn_stream_t s);
+
+/* win x win max-pool (stride, zero-free padding: out-of-image taps are ignored) over uint8 codes
+ * [B][H][W][C], then bit-plane packing with the Bit_compression layout (NN/kernel.cuh:46-77):
+ * planes:[bits][B*Ho*Wo][cpad/32].  win = stride = 1, pad = 0 packs without pooling. */
+int apnn_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits, int win,
+                   int stride, int pad, apnn_stream_t s);
+
+/* Packed codes -> int8: out[r][c] = min(127, (sum_{j<group} code[r*group+j][c]) >> shift).
+ * group = 1, shift = 0 unpacks (inverse of the packer, cf. UnpackConvOutput32, NN/param.h:634-658);
+ * group = H*W pools a feature map globally.  planes:[bits][rows_out*group][cpad/32]. */
+int apnn_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad, int bits,
+                    int shift, apnn_stream_t s);
+
+/* int8 classifier with a float affine output, out[b][n] = scale[n]*sum_k X[b][k]*Wt[n][k] + bias[n]
+ * (the output layer's  val*bn_scale + bn_bias, NN/kernel.cuh:437-441).  acc_out (optional) receives
+ * the int32 sums. */
+int apnn_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
+               int32_t *acc_out, int B, int N, int K, apnn_stream_t s);
 
 /* Library / device information: number of compute units of the current device (0 if none). */
 int apnn_device_cus(void);

@@ -34,13 +34,16 @@ def to_host(t, dtype=np.int32):
     return a.view(dtype) if dtype != a.dtype else a
 
 
-def epilogue(mode=0, out_bits=0, pool=0, thr=None, flip=None, resid=None, save=None):
+def epilogue(mode=0, out_bits=0, pool=0, thr=None, flip=None, resid=None, save=None, resid_planes=None,
+             resid_bits=0, resid_scale=0):
     e = A.Epilogue()
     e.mode, e.out_bits, e.pool = mode, out_bits, pool
     e.thresholds = thr.data_ptr() if thr is not None else None
     e.flip = flip.data_ptr() if flip is not None else None
     e.residual = resid.data_ptr() if resid is not None else None
     e.save_acc = save.data_ptr() if save is not None else None
+    e.residual_planes = resid_planes.data_ptr() if resid_planes is not None else None
+    e.residual_bits, e.residual_scale = resid_bits, resid_scale
     return e
 
 

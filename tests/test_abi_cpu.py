@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_sizes_match_header_layout():
     # 3 ints (+pad) + 4 pointers; keeps the ctypes mirror honest about field order
-    assert ctypes.sizeof(A.Epilogue) == 16 + 4 * 8
+    assert ctypes.sizeof(A.Epilogue) == 16 + 5 * 8 + 8
     assert A.GemmDesc.epi.offset == 3 * 8 + 6 * 4
     assert A.ConvDesc.epi.offset == 3 * 8 + 13 * 4 + 4
 

@@ -284,3 +284,97 @@ def test_gemm_2048_sampled_and_closed_form(G, wb, xb, path):
     ones_w = np.full_like(W, 0xFFFFFFFF)
     ones_x = np.full_like(X, 0xFFFFFFFF)
     assert np.all(G.run_gemm(ones_w, ones_x, M, N, K, wb, xb, path=path) == K * (2 ** wb - 1) * (2 ** xb - 1))
+
+
+# ---- layers on either side of the low-bit path ---------------------------------------------------
+
+def _np_maxpool_codes(codes, win, stride, pad):
+    B, H, W, C = codes.shape
+    Ho, Wo = (H + 2 * pad - win) // stride + 1, (W + 2 * pad - win) // stride + 1
+    padded = np.zeros((B, H + 2 * pad, W + 2 * pad, C), codes.dtype)     # codes are >= 0: zero padding == ignoring
+    padded[:, pad:pad + H, pad:pad + W] = codes
+    out = np.zeros((B, Ho, Wo, C), codes.dtype)
+    for r in range(win):
+        for s in range(win):
+            out = np.maximum(out, padded[:, r:r + stride * (Ho - 1) + 1:stride, s:s + stride * (Wo - 1) + 1:stride])
+    return out
+
+
+@pytest.mark.parametrize("R,stride,pad,H,cout", [(7, 2, 3, 32, 64), (11, 4, 5, 35, 64), (3, 1, 1, 9, 40)])
+def test_conv_i8_bn_and_pool_pack(G, R, stride, pad, H, cout):
+    rng = np.random.default_rng(900 + R)
+    B, C, bits = 2, 3, 2
+    X = rng.integers(-128, 128, size=(B, H, H, C)).astype(np.int8)
+    Wt = rng.integers(-128, 128, size=(cout, R, R, C)).astype(np.int8)
+    acc = O.conv_i8(Wt, X, stride, pad)
+    Ho = acc.shape[1]
+    thr = np.sort(rng.integers(-60000, 60000, size=(cout, 3)), axis=1).astype(np.int32)
+    dX, dW, dT = G.to_dev(X), G.to_dev(Wt), G.to_dev(thr)
+    d_codes = torch.empty(B * Ho * Ho * cout, dtype=torch.uint8, device="cuda")
+    d_acc = G.dev_empty_i32(B * Ho * Ho * cout, fill=-7)
+    L = G.A.lib()
+    G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, H, C, cout, R, R,
+                                stride, pad, bits, None), "conv_i8_bn")
+    assert np.array_equal(G.to_host(d_acc).reshape(acc.shape), acc)
+    codes = O.bn_quantize(acc.reshape(-1, cout), None, thr, None, bits).reshape(acc.shape).astype(np.uint8)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_codes.cpu().numpy().reshape(acc.shape), codes)
+    for win, st, pd in [(3, 2, 1), (2, 2, 0), (1, 1, 0)]:
+        pooled = _np_maxpool_codes(codes, win, st, pd)
+        rows = pooled.shape[0] * pooled.shape[1] * pooled.shape[2]
+        cpad = 128
+        d_planes = G.dev_empty_i32(bits * rows * cpad // 32, fill=-7)
+        G.A.check(L.apnn_pool_pack(G.ptr(d_codes), G.ptr(d_planes), B, Ho, Ho, cout, cpad, bits, win, st, pd, None),
+                  "pool_pack")
+        expect = O.pack_bits(pooled.reshape(rows, cout).astype(np.uint32), rows, cout, cpad, bits)
+        assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect)
+
+
+def test_unpack_sum_and_fc_i8(G):
+    rng = np.random.default_rng(950)
+    B, HW, C, cpad, bits, N = 4, 49, 200, 256, 2, 37
+    codes = rng.integers(0, 4, size=(B * HW, C)).astype(np.uint32)
+    planes = O.pack_bits(codes, B * HW, C, cpad, bits)
+    d_planes = G.to_dev(planes)
+    L = G.A.lib()
+    d_un = torch.empty(B * HW * C, dtype=torch.int8, device="cuda")
+    G.A.check(L.apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_un), B * HW, 1, C, cpad, bits, 0, None), "unpack")
+    torch.cuda.synchronize()
+    assert np.array_equal(d_un.cpu().numpy().reshape(B * HW, C), codes.astype(np.int8))
+    d_pool = torch.empty(B * C, dtype=torch.int8, device="cuda")
+    G.A.check(L.apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_pool), B, HW, C, cpad, bits, 1, None), "pool")
+    torch.cuda.synchronize()
+    pooled = np.minimum(127, codes.reshape(B, HW, C).sum(1) >> 1).astype(np.int8)
+    assert np.array_equal(d_pool.cpu().numpy().reshape(B, C), pooled)
+    Wt = rng.integers(-128, 128, size=(N, C)).astype(np.int8)
+    scale = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    d_out = torch.empty(B * N, dtype=torch.float32, device="cuda")
+    d_acc = G.dev_empty_i32(B * N, fill=-7)
+    dW, dS, dB = G.to_dev(Wt), torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
+    G.A.check(L.apnn_fc_i8(G.ptr(d_pool), G.ptr(dW), G.ptr(dS), G.ptr(dB), G.ptr(d_out), G.ptr(d_acc), B, N, C, None), "fc")
+    acc = pooled.astype(np.int64) @ Wt.astype(np.int64).T
+    assert np.array_equal(G.to_host(d_acc).reshape(B, N), acc)
+    torch.cuda.synchronize()
+    # float affine of an exact int32: one fp32 multiply-add, tolerance 1e-6 relative
+    expect = acc.astype(np.float32) * scale[None, :] + bias[None, :]
+    assert np.allclose(d_out.cpu().numpy().reshape(B, N), expect, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("path", PATHS)
+def test_conv_packed_residual(G, path):
+    """Identity shortcut: the block input's packed codes are added, scaled, before the thresholds."""
+    rng = np.random.default_rng(970 + path)
+    batch, H, Wd, C, wb, xb, ob = 2, 14, 14, 128, 1, 2, 2
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, C * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw).reshape(-1, C)
+    short = rng.integers(0, 4, size=acc.shape).astype(np.uint32)
+    short_planes = O.pack_bits(short, acc.shape[0], C, C, 2)
+    thr = np.sort(rng.integers(-100, 100, size=(C, 3)), axis=1).astype(np.int32)
+    d_thr, d_sp = G.to_dev(thr), G.to_dev(short_planes)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, resid_planes=d_sp, resid_bits=2, resid_scale=24)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, **kw).view(np.uint32).reshape(ob, -1, C // 32)
+    q = O.bn_quantize(acc + 24 * short.astype(np.int32), None, thr, None, ob)
+    assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
