@@ -13,4 +13,8 @@ Python is only a convenience for tests and benchmarks; the product is the C ABI 
 include/apnn_tc.h.  There is no CPU fallback: every call goes to the HIP library.
 """
 from .binding import *  # noqa: F401,F403
-from .binding import __all__  # noqa: F401
+from .binding import __all__ as _b_all
+from .nn_binding import *  # noqa: F401,F403
+from .nn_binding import __all__ as _n_all
+
+__all__ = list(_b_all) + list(_n_all)

@@ -102,7 +102,7 @@ def lib():
         L.apnn_conv.restype = _ci
         L.apnn_pack_bits.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]
         L.apnn_pack_bits.restype = _ci
-        L.apnn_conv_i8_bn.argtypes = [_vp] * 5 + [_ci] * 10 + [_vp]
+        L.apnn_conv_i8_bn.argtypes = [_vp] * 5 + [_ci] * 11 + [_vp]
         L.apnn_conv_i8_bn.restype = _ci
         L.apnn_pool_pack.argtypes = [_vp, _vp] + [_ci] * 9 + [_vp]
         L.apnn_pool_pack.restype = _ci

@@ -349,16 +349,17 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
 
 int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint8_t *codes, int32_t *acc_out,
                     int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
-                    apnn_stream_t s) {
+                    int x_zero_point, apnn_stream_t s) {
   if (X == nullptr || Wt == nullptr || (codes == nullptr && acc_out == nullptr)) return APNN_ENULL;
   if (codes != nullptr && thresholds == nullptr) return APNN_ENULL;
   if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || COUT <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0)
     return APNN_EINVAL;
   if (H + 2 * pad < R || W + 2 * pad < S) return APNN_EINVAL;
   if (codes != nullptr && (bits < 1 || bits > 8)) return APNN_EINVAL;
+  if (x_zero_point < 0 || x_zero_point > 255) return APNN_EINVAL;
   if ((long long)64 * R * S * C > 64 * 1024) return APNN_EUNSUPPORTED;  // filter block must fit in LDS
   return (int)apnn::launch_conv_i8_bn(X, Wt, thresholds, codes, acc_out, B, H, W, C, COUT, R, S, stride, pad, bits,
-                                      static_cast<hipStream_t>(s));
+                                      x_zero_point, static_cast<hipStream_t>(s));
 }
 
 int apnn_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits, int win,

@@ -9,7 +9,8 @@
 namespace apnn {
 
 // ---- int8 first convolution + per-channel thresholds -> codes ------------------------------------
-// X: [B][H][W][C] int8, Wt: [COUT][R][S][C] int8 (C tiny: 3), thr: [COUT][2^bits-1] int32.
+// X: [B][H][W][C] int8 (or uint8 minus zero_point when zero_point != 0), Wt: [COUT][R][S][C] int8
+// (C tiny: 3), thr: [COUT][2^bits-1] int32.
 // One work-group computes a strip of 64 output pixels x COUT_T=64 channels; the filter block is
 // staged in LDS once, each thread owns one pixel and 16 channels.
 template <int COUT_T>
@@ -17,7 +18,7 @@ __global__ __launch_bounds__(256) void conv_i8_bn_kernel(const int8_t *__restric
                                                          const int32_t *__restrict__ thr,
                                                          uint8_t *__restrict__ codes, int32_t *__restrict__ acc_out,
                                                          int B, int H, int W, int C, int COUT, int R, int S,
-                                                         int stride, int pad, int Ho, int Wo, int bits) {
+                                                         int stride, int pad, int Ho, int Wo, int bits, int zero_point) {
   extern __shared__ int8_t wlds[];  // [COUT_T][R*S*C]
   const int K = R * S * C;
   const int co0 = blockIdx.y * COUT_T;
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(256) void conv_i8_bn_kernel(const int8_t *__restric
       const int8_t *xp = X + (((long long)b * H + iy) * W + ix) * C;
       const int8_t *wp = wlds + (cg * 16) * K + (r * S + s) * C;
       for (int c = 0; c < C; ++c) {
-        const int xv = xp[c];
+        const int xv = zero_point ? (int)(uint8_t)xp[c] - zero_point : (int)xp[c];
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[j] += xv * (int)wp[j * K + c];
       }
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restr
 }
 
 // ---- int8 classifier: out[b][n] = scale[n] * sum_k X[b][k] * Wt[n][k] + bias[n] -----------------
-// One wave per output; K % 4 == 0 handled by 4-byte dot products, tail by bytes.
+// One wave per output: lanes stride over K, then a wave64 butterfly reduction.
 __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                     const float *__restrict__ scale, const float *__restrict__ bias,
                                                     float *__restrict__ out, int32_t *__restrict__ acc_out, int Bn,
@@ -151,13 +152,13 @@ __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X
 
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
                              int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
-                             hipStream_t s) {
+                             int zero_point, hipStream_t s) {
   const int Ho = (H + 2 * pad - R) / stride + 1, Wo = (W + 2 * pad - S) / stride + 1;
   const long long npix = (long long)B * Ho * Wo;
   const size_t lds = (size_t)64 * R * S * C;
   dim3 grid((unsigned)((npix + 63) / 64), (unsigned)((COUT + 63) / 64));
   hipLaunchKernelGGL(conv_i8_bn_kernel<64>, grid, dim3(256), lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT, R,
-                     S, stride, pad, Ho, Wo, bits);
+                     S, stride, pad, Ho, Wo, bits, zero_point);
   return hipGetLastError();
 }
 

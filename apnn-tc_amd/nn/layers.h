@@ -1,0 +1,201 @@
+// Layer API of the low-bit network path: host-side C++ classes with the names, constructor
+// arguments and life cycle (constructor -> initialize() -> forward -> download_output() -> release())
+// of the reference's layer parameter classes in APNN-TC-nn/src/param.h, driven through the C ABI of
+// libapnn_tc.so.  Differences that are deliberate:
+//   * a layer object stays on the host (the reference copies it to the device and hands the device
+//     pointer to a kernel, param.h:949-960); the *_new_global wrappers take the host object and a
+//     stream and enqueue the kernels;
+//   * batch-norm is folded into 2^a-1 per-channel integer thresholds (the reference's layers have a
+//     single float threshold, usable for 1-bit outputs only, kernel.cuh:833-834);
+//   * the shortcut of a residual block is the packed output of an earlier layer, added at an integer
+//     scale inside the epilogue;
+//   * weights and thresholds are random-initialised from a seeded generator (the reference reads a
+//     CSV through launch_array, which is disabled: utility.h:174-182).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/apnn_nn.h"
+#include "../../include/apnn_tc.h"
+
+namespace apnn_nn {
+
+inline int pad_to(int x, int m) { return (x + m - 1) / m * m; }
+
+// splitmix64: seeded, platform independent
+struct Rng {
+  uint64_t s;
+  explicit Rng(uint64_t seed) : s(seed) {}
+  uint64_t next() {
+    uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+  }
+  uint32_t below(uint32_t n) { return (uint32_t)((next() >> 32) * (uint64_t)n >> 32); }
+  double uniform() { return (double)(next() >> 11) * (1.0 / 9007199254740992.0); }
+};
+
+// device allocation owned by a layer
+class DeviceBuffer {
+ public:
+  DeviceBuffer() = default;
+  ~DeviceBuffer() { release(); }
+  DeviceBuffer(const DeviceBuffer &) = delete;
+  DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+  hipError_t allocate(size_t bytes);
+  hipError_t upload(const void *host, size_t bytes);
+  void release();
+  void *get() const { return ptr_; }
+  size_t bytes() const { return bytes_; }
+  template <class T> T *as() const { return static_cast<T *>(ptr_); }
+
+ private:
+  void *ptr_ = nullptr;
+  size_t bytes_ = 0;
+};
+
+class Layer {
+ public:
+  virtual ~Layer() = default;
+  virtual int forward(hipStream_t stream) = 0;
+  virtual void describe(apnn_layer_desc *d) const = 0;
+  virtual const uint32_t *get_output_gpu() const { return nullptr; }
+};
+
+// First layer: int8 convolution on uint8 pixels (zero point 128), thresholds -> a-bit codes,
+// optional max-pool, bit-plane packing.  Counterpart of InConv128LayerParam (param.h:701-875), which
+// binarises a float image convolution; the int8 arithmetic follows cutlass_nn/src/config.h:215-255.
+class InConv128LayerParam : public Layer {
+ public:
+  InConv128LayerParam(const char *name, int input_height, int input_width, int filter_height, int filter_width,
+                      int input_channels, int output_channels, int batch, int stride_height = 1,
+                      int stride_width = 1, bool padding = true, int pool_height = 1, int pool_width = 1,
+                      int pool_stride = 0, int pool_pad = 0, int a_bit = 2);
+  int initialize(Rng &rng, const uint8_t *images_gpu);
+  void set_input_gpu(const uint8_t *images_gpu) { input_gpu = images_gpu; }
+  int forward(hipStream_t stream) override;
+  void describe(apnn_layer_desc *d) const override;
+  const uint32_t *get_output_gpu() const override { return output_gpu.as<uint32_t>(); }
+  std::vector<uint32_t> download_output() const;
+
+  std::string name;
+  int input_height, input_width, filter_height, filter_width, input_channels, output_channels, batch;
+  int stride, pad, pool, pool_stride, pool_pad, a_bit;
+  int conv_height, conv_width, output_height, output_width, out_cpad;
+  const uint8_t *input_gpu = nullptr;
+  DeviceBuffer filter_gpu, bn_gpu, codes_gpu, output_gpu;
+};
+
+// Low-bit convolution layer (param.h:877-1083).  pool_height == 2 applies a 2x2 max-pool to the
+// quantized codes inside the epilogue.  inject_residual adds `residual_scale` x the packed codes of
+// the shortcut layer before the thresholds.
+class Conv128LayerParam : public Layer {
+ public:
+  Conv128LayerParam(const char *name, int input_height, int input_width, int filter_height, int filter_width,
+                    int input_channels, int output_channels, int batch, int stride_height = 1, int stride_width = 1,
+                    bool padding = true, int pool_height = 1, int pool_width = 1, bool ahead_fc = false,
+                    bool save_residual = false, bool inject_residual = false, int residual_channels = 0,
+                    bool residual_pool = false, int a_bit = 2, int w_bit = 1);
+  // sizes in the reference's terms (param.h:927-945), for this layout (channels padded to in_cpad)
+  long long input_bit_words() const { return (long long)a_bit * batch * input_height * input_width * (in_cpad / 32); }
+  long long filter_bit_words() const {
+    return (long long)w_bit * output_channels * filter_height * filter_width * (in_cpad / 32);
+  }
+  long long output_bit_words() const {
+    return (long long)a_bit * batch * output_height * output_width * (out_cpad / 32);
+  }
+  int initialize(Rng &rng, const uint32_t *prev_layer_gpu, const uint32_t *input_residual_gpu = nullptr,
+                 int residual_scale = 0, int path = APNN_PATH_AUTO);
+  void set_input_gpu(const uint32_t *p) { input_gpu = p; }
+  int forward(hipStream_t stream) override;
+  void describe(apnn_layer_desc *d) const override;
+  const uint32_t *get_output_gpu() const override { return output_gpu.as<uint32_t>(); }
+  std::vector<uint32_t> download_output() const;
+
+  std::string name;
+  int input_height, input_width, filter_height, filter_width, input_channels, output_channels, batch;
+  int stride, pad, pool, a_bit, w_bit;
+  bool inject_residual;
+  int conv_height, conv_width, output_height, output_width, in_cpad, out_cpad;
+  int residual_scale = 0, path = APNN_PATH_AUTO, shortcut_layer = -1;
+  const uint32_t *input_gpu = nullptr, *input_residual_gpu = nullptr;
+  DeviceBuffer filter_gpu, bn_gpu, output_gpu;
+};
+
+// Low-bit fully connected layer (param.h:219-385): rows = batch, a convolution whose filter spans the
+// whole (in_h x in_w) input map, so the NHWC feature map of the previous layer is consumed as is.
+class Fc128LayerParam : public Layer {
+ public:
+  Fc128LayerParam(const char *name, int batch, int input_height, int input_width, int input_channels,
+                  int weight_width, int a_bit = 2, int w_bit = 1);
+  int initialize(Rng &rng, const uint32_t *prev_layer_gpu, int path = APNN_PATH_AUTO);
+  int forward(hipStream_t stream) override;
+  void describe(apnn_layer_desc *d) const override;
+  const uint32_t *get_output_gpu() const override { return output_gpu.as<uint32_t>(); }
+
+  std::string name;
+  int batch, input_height, input_width, input_channels, weight_width, a_bit, w_bit;
+  int in_cpad, out_cpad, path = APNN_PATH_AUTO;
+  const uint32_t *input_gpu = nullptr;
+  DeviceBuffer weight_gpu, bn_gpu, output_gpu;
+};
+
+// Output layer (param.h:388-531): the packed codes of the previous layer are unpacked (optionally
+// summed over the feature map: global average pooling up to a shift) to int8 and multiplied by an
+// int8 weight matrix; logits = acc * bn_scale + bn_bias in float (kernel.cuh:437-441).
+class Out128LayerParam : public Layer {
+ public:
+  Out128LayerParam(const char *name, int batch, int input_positions, int input_channels, int weight_width,
+                   int global_pool_shift, int a_bit = 2);
+  int initialize(Rng &rng, const uint32_t *prev_layer_gpu, float *logits_gpu);
+  void set_output_gpu(float *logits) { output_gpu = logits; }
+  int forward(hipStream_t stream) override;
+  void describe(apnn_layer_desc *d) const override;
+
+  std::string name;
+  int batch, input_positions, input_channels, weight_width, global_pool_shift, a_bit, in_cpad;
+  const uint32_t *input_gpu = nullptr;
+  float *output_gpu = nullptr;
+  DeviceBuffer weight_gpu, scale_gpu, bias_gpu, pooled_gpu;
+};
+
+// Launch wrappers with the reference's names (kernel.cuh:285-318): unpack the layer object into the
+// kernel call.  The reference launches a __global__ wrapper around a __device__ kernel; here the
+// wrapper is a host function that enqueues on `stream`.
+int Conv_new_global(Conv128LayerParam *p, hipStream_t stream);
+int FC_new_global(Fc128LayerParam *p, hipStream_t stream);
+int Output_new_global(Out128LayerParam *p, hipStream_t stream);
+
+// Random codes -> bit-planes on the device with the layout of filter_quantization /
+// weight_quantization (kernel.cuh:164-282): values [rows][C] uniform in [0, 2^bits), packed with
+// apnn_pack_bits (Bit_compression layout), pad channels zero.
+int random_planes_gpu(Rng &rng, DeviceBuffer &planes, int rows, int C, int cpad, int bits);
+// Thresholds [C][2^bits-1] around `center` with spread sigma (quartile-like spacing + jitter).
+std::vector<int32_t> random_thresholds(Rng &rng, int C, int bits, double center, double sigma);
+
+class Network {
+ public:
+  ~Network();
+  int forward(const uint8_t *images, float *logits, hipStream_t stream);
+  int forward_graph(const uint8_t *images, float *logits, hipStream_t stream);
+  std::vector<std::unique_ptr<Layer>> layers;
+  InConv128LayerParam *first = nullptr;
+  Out128LayerParam *last = nullptr;
+  int batch = 0;
+
+ private:
+  hipGraphExec_t graph_exec_ = nullptr;
+  hipStream_t capture_stream_ = nullptr;
+  const uint8_t *graph_images_ = nullptr;
+  float *graph_logits_ = nullptr;
+};
+
+std::unique_ptr<Network> build_alexnet(int batch, uint64_t seed, int path);
+std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path);
+
+}  // namespace apnn_nn

@@ -1,0 +1,158 @@
+// Network builders (the counterparts of the reference's demo drivers) and the C ABI of
+// libapnn_nn.so.  See include/apnn_nn.h.
+#include <cmath>
+#include <new>
+
+#include "layers.h"
+
+namespace apnn_nn {
+
+namespace {
+
+// shortcut codes (0..amax) are brought to roughly half a standard deviation of the main branch
+int shortcut_scale_for(int filter_h, int filter_w, int cin, int a_bit) {
+  const double amax = (double)((1 << a_bit) - 1);
+  const double sigma = std::sqrt((double)filter_h * filter_w * cin * amax * (2 * amax + 1) / 6.0);
+  const int s = (int)std::lround(sigma / (2.0 * amax));
+  return s < 1 ? 1 : s;
+}
+
+template <class L>
+L *add(Network &net, L *layer) {
+  net.layers.emplace_back(layer);
+  return layer;
+}
+
+}  // namespace
+
+// AlexNet-style network, layer list of APNN-TC-nn/src/alexnet.cu:42-81: conv 11x11/4 3->64 pool 2,
+// conv 5x5 64->192 pool 2, conv 3x3 192->384, 384->256, 256->256 pool 2, FC 12544->4096->4096->1000.
+// First conv and classifier in int8, hidden layers w1a2.
+std::unique_ptr<Network> build_alexnet(int batch, uint64_t seed, int path) {
+  auto net = std::make_unique<Network>();
+  net->batch = batch;
+  Rng rng(seed);
+  auto *c1 = add(*net, new InConv128LayerParam("Conv1", 224, 224, 11, 11, 3, 64, batch, 4, 4, true, 2, 2));
+  if (c1->initialize(rng, nullptr)) return nullptr;
+  net->first = c1;
+  auto *c2 = add(*net, new Conv128LayerParam("Conv2", c1->output_height, c1->output_width, 5, 5, 64, 192, batch, 1, 1,
+                                             true, 2, 2));
+  if (c2->initialize(rng, c1->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  auto *c3 = add(*net, new Conv128LayerParam("Conv3", c2->output_height, c2->output_width, 3, 3, 192, 384, batch));
+  if (c3->initialize(rng, c2->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  auto *c4 = add(*net, new Conv128LayerParam("Conv4", c3->output_height, c3->output_width, 3, 3, 384, 256, batch));
+  if (c4->initialize(rng, c3->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  auto *c5 = add(*net, new Conv128LayerParam("Conv5", c4->output_height, c4->output_width, 3, 3, 256, 256, batch, 1, 1,
+                                             true, 2, 2));
+  if (c5->initialize(rng, c4->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, c5->output_height, c5->output_width, 256, 4096));
+  if (f1->initialize(rng, c5->get_output_gpu(), path)) return nullptr;
+  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 1, 1, 4096, 4096));
+  if (f2->initialize(rng, f1->get_output_gpu(), path)) return nullptr;
+  auto *out = add(*net, new Out128LayerParam("Fout", batch, 1, 4096, 1000, -1));
+  if (out->initialize(rng, f2->get_output_gpu(), nullptr)) return nullptr;
+  net->last = out;
+  return net;
+}
+
+// Standard ResNet18: 7x7/2 int8 stem + 3x3/2 max-pool, four stages of two basic blocks at
+// 64/128/256/512 channels, a strided 1x1 convolution on the shortcut where the shape changes, global
+// average pool and an int8 classifier.  (The reference's own demo, APNN-TC-nn/src/resnet18.cu:40-142,
+// uses a stride-4 stem and pooled int32 residuals instead of 1x1 convolutions.)
+std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path) {
+  auto net = std::make_unique<Network>();
+  net->batch = batch;
+  Rng rng(seed);
+  auto *stem = add(*net, new InConv128LayerParam("Conv1", 224, 224, 7, 7, 3, 64, batch, 2, 2, true, 3, 3, 2, 1));
+  if (stem->initialize(rng, nullptr)) return nullptr;
+  net->first = stem;
+  const uint32_t *prev = stem->get_output_gpu();
+  int prev_index = 0;
+  int h = stem->output_height, w = stem->output_width, cin = 64;
+  for (int stage = 0; stage < 4; ++stage) {
+    const int ch = 64 << stage;
+    for (int blk = 0; blk < 2; ++blk) {
+      const int stride = (stage > 0 && blk == 0) ? 2 : 1;
+      char nm[16];
+      snprintf(nm, sizeof nm, "L%dB%dC1", stage + 1, blk + 1);
+      auto *c1 = add(*net, new Conv128LayerParam(nm, h, w, 3, 3, cin, ch, batch, stride, stride));
+      if (c1->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+      const uint32_t *shortcut = prev;
+      int shortcut_index = prev_index;
+      if (stride != 1 || cin != ch) {
+        snprintf(nm, sizeof nm, "L%dB%dDS", stage + 1, blk + 1);
+        auto *ds = add(*net, new Conv128LayerParam(nm, h, w, 1, 1, cin, ch, batch, stride, stride, false));
+        if (ds->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+        shortcut = ds->get_output_gpu();
+        shortcut_index = (int)net->layers.size() - 1;
+      }
+      snprintf(nm, sizeof nm, "L%dB%dC2", stage + 1, blk + 1);
+      auto *c2 = add(*net, new Conv128LayerParam(nm, c1->output_height, c1->output_width, 3, 3, ch, ch, batch, 1, 1,
+                                                 true, 1, 1, false, false, true, ch));
+      if (c2->initialize(rng, c1->get_output_gpu(), shortcut, shortcut_scale_for(3, 3, ch, 2), path)) return nullptr;
+      c2->shortcut_layer = shortcut_index;
+      prev = c2->get_output_gpu();
+      prev_index = (int)net->layers.size() - 1;
+      h = c2->output_height;
+      w = c2->output_width;
+      cin = ch;
+    }
+  }
+  auto *out = add(*net, new Out128LayerParam("Fc", batch, h * w, 512, 1000, 1));
+  if (out->initialize(rng, prev, nullptr)) return nullptr;
+  net->last = out;
+  return net;
+}
+
+}  // namespace apnn_nn
+
+struct apnn_net {
+  std::unique_ptr<apnn_nn::Network> impl;
+};
+
+extern "C" {
+
+apnn_net *apnn_net_create(int kind, int batch, unsigned long long seed, int path) {
+  if (batch <= 0) return nullptr;
+  std::unique_ptr<apnn_nn::Network> n;
+  if (kind == APNN_NET_ALEXNET) {
+    n = apnn_nn::build_alexnet(batch, seed, path);
+  } else if (kind == APNN_NET_RESNET18) {
+    n = apnn_nn::build_resnet18(batch, seed, path);
+  }
+  if (!n) return nullptr;
+  apnn_net *h = new (std::nothrow) apnn_net;
+  if (h == nullptr) return nullptr;
+  h->impl = std::move(n);
+  return h;
+}
+
+void apnn_net_destroy(apnn_net *net) { delete net; }
+
+int apnn_net_forward(apnn_net *net, const uint8_t *images, float *logits, apnn_stream_t s) {
+  if (net == nullptr) return APNN_ENULL;
+  return net->impl->forward(images, logits, static_cast<hipStream_t>(s));
+}
+
+int apnn_net_forward_graph(apnn_net *net, const uint8_t *images, float *logits, apnn_stream_t s) {
+  if (net == nullptr) return APNN_ENULL;
+  return net->impl->forward_graph(images, logits, static_cast<hipStream_t>(s));
+}
+
+int apnn_net_layer_count(const apnn_net *net) { return net == nullptr ? 0 : (int)net->impl->layers.size(); }
+
+int apnn_net_layer(const apnn_net *net, int index, apnn_layer_desc *out) {
+  if (net == nullptr || out == nullptr) return APNN_ENULL;
+  if (index < 0 || index >= (int)net->impl->layers.size()) return APNN_EINVAL;
+  net->impl->layers[index]->describe(out);
+  return APNN_OK;
+}
+
+int apnn_nn_download(void *host_dst, const void *dev_src, unsigned long long bytes) {
+  if (host_dst == nullptr || dev_src == nullptr) return APNN_ENULL;
+  hipError_t e = hipDeviceSynchronize();
+  if (e != hipSuccess) return (int)e;
+  return (int)hipMemcpy(host_dst, dev_src, bytes, hipMemcpyDeviceToHost);
+}
+
+}  // extern "C"

@@ -1,0 +1,72 @@
+/*
+ * apnn_nn.h -- C view of the network layer (libapnn_nn.so), the counterpart of the reference's
+ * APNN-TC-nn demo drivers (APNN-TC-nn/src/alexnet.cu, resnet18.cu) and layer classes
+ * (APNN-TC-nn/src/param.h).  The C++ classes themselves (Conv128LayerParam, Fc128LayerParam,
+ * Out128LayerParam, InConv128LayerParam and the *_new_global wrappers) are declared in
+ * apnn-tc_amd/nn/layers.h; this header is what a non-C++ host (tests, benchmark) binds.
+ *
+ * A network owns its device buffers (weights, thresholds, activations); forward() only enqueues
+ * kernels on the given stream: no allocation, no host synchronisation between layers.
+ */
+#ifndef APNN_NN_H
+#define APNN_NN_H
+
+#include <stdint.h>
+
+#include "apnn_tc.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { APNN_NET_ALEXNET = 0,   /* topology of APNN-TC-nn/src/alexnet.cu:42-81, int8 first conv / classifier */
+       APNN_NET_RESNET18 = 1 };/* standard ResNet18 (3x3 basic blocks, strided 1x1 downsample convs)        */
+
+enum { APNN_LAYER_INCONV_I8 = 0, /* int8 conv + thresholds (+ max-pool) + pack                               */
+       APNN_LAYER_CONV = 1,      /* low-bit conv, fused threshold / pool / shortcut epilogue                  */
+       APNN_LAYER_FC = 2,        /* low-bit fully connected (a conv whose filter covers its whole input)      */
+       APNN_LAYER_OUT_I8 = 3 };  /* (global pool +) int8 classifier, float logits                             */
+
+typedef struct apnn_layer_desc {
+  char name[16];
+  int kind;
+  int batch;
+  int in_h, in_w, in_c, in_cpad;       /* input feature map (cpad = stored channels) */
+  int out_h, out_w, out_c, out_cpad;   /* output after pooling */
+  int R, S, stride, pad;
+  int pool_win, pool_stride, pool_pad; /* max-pool applied to the quantized codes (0 = none) */
+  int a_bits, w_bits, out_bits;
+  int shortcut_layer;                  /* index of the layer whose packed output is the shortcut, -1 none */
+  int shortcut_scale;
+  int global_pool_shift;               /* OUT_I8: pooled = min(127, sum_of_codes >> shift); -1: no pooling */
+  const void *input;                   /* device pointers, valid for the lifetime of the network */
+  const void *weights;                 /* CONV/FC: packed planes [w][cout][R][S][in_cpad/32]; I8: [cout][R][S][in_c] */
+  const void *thresholds;              /* [out_c][2^out_bits-1] int32 */
+  const void *scale, *bias;            /* OUT_I8: float [out_c] */
+  const void *output;                  /* packed planes [out_bits][batch*out_h*out_w][out_cpad/32]; OUT_I8: float */
+} apnn_layer_desc;
+
+typedef struct apnn_net apnn_net;
+
+/* Builds the network with random-init weights / thresholds from `seed`.  path: APNN_PATH_* for the
+ * low-bit layers.  Returns NULL on failure. */
+apnn_net *apnn_net_create(int kind, int batch, unsigned long long seed, int path);
+void apnn_net_destroy(apnn_net *net);
+
+/* images: device, [batch][224][224][3] uint8; logits: device, [batch][1000] float. */
+int apnn_net_forward(apnn_net *net, const uint8_t *images, float *logits, apnn_stream_t s);
+
+/* Records forward() into a HIP graph once (on an internal capture stream) and replays it with a
+ * single launch per call: removes the per-kernel launch gaps of a 20-layer network. */
+int apnn_net_forward_graph(apnn_net *net, const uint8_t *images, float *logits, apnn_stream_t s);
+
+int apnn_net_layer_count(const apnn_net *net);
+int apnn_net_layer(const apnn_net *net, int index, apnn_layer_desc *out);
+
+/* Blocking device-to-host copy for buffers owned by a network. */
+int apnn_nn_download(void *host_dst, const void *dev_src, unsigned long long bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -164,10 +164,11 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
  * cutlass_nn/src/config.h:215-255: int8 operands, int32 accumulate), followed by per-channel
  * thresholds: code = #{k : acc >= thresholds[c][k]}.
  * X:[B][H][W][C] int8, Wt:[COUT][R][S][C] int8; codes:[B][Ho][Wo][COUT] uint8 (NULL to skip),
- * acc_out:[B][Ho][Wo][COUT] int32 (NULL to skip); thresholds may be NULL when codes is NULL. */
+ * acc_out:[B][Ho][Wo][COUT] int32 (NULL to skip); thresholds may be NULL when codes is NULL.
+ * x_zero_point != 0: X holds uint8 pixels and x - x_zero_point is convolved (128 for raw images). */
 int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint8_t *codes, int32_t *acc_out,
                     int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
-                    apnn_stream_t s);
+                    int x_zero_point, apnn_stream_t s);
 
 /* win x win max-pool (stride, zero-free padding: out-of-image taps are ignored) over uint8 codes
  * [B][H][W][C], then bit-plane packing with the Bit_compression layout (NN/kernel.cuh:46-77):

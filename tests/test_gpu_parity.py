@@ -314,7 +314,7 @@ def test_conv_i8_bn_and_pool_pack(G, R, stride, pad, H, cout):
     d_acc = G.dev_empty_i32(B * Ho * Ho * cout, fill=-7)
     L = G.A.lib()
     G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, H, C, cout, R, R,
-                                stride, pad, bits, None), "conv_i8_bn")
+                                stride, pad, bits, 0, None), "conv_i8_bn")
     assert np.array_equal(G.to_host(d_acc).reshape(acc.shape), acc)
     codes = O.bn_quantize(acc.reshape(-1, cout), None, thr, None, bits).reshape(acc.shape).astype(np.uint8)
     torch.cuda.synchronize()
