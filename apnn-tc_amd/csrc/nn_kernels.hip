@@ -67,6 +67,108 @@ __global__ __launch_bounds__(256) void conv_i8_bn_kernel(const int8_t *__restric
   }
 }
 
+// ---- int8 first convolution on the matrix cores ------------------------------------------------------
+// Implicit GEMM: rows = 32 consecutive output pixels of one output row (one wave), columns = 64 output
+// channels (two 32x32 blocks), K = R*S*C rounded up to k-steps of 32 with v_mfma_i32_32x32x32_i8.
+// The filter block [64][T*32] (zero padded) and, per wave, the input patch that the 32 pixels touch
+// (R rows x ((31*stride + S) * C) bytes, already minus the zero point, zero outside the image) sit in
+// LDS; a small table maps k -> (patch row offset) so that any R, S, C works.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void conv_i8_mfma_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                           const int32_t *__restrict__ thr,
+                                                           uint8_t *__restrict__ codes, int32_t *__restrict__ acc_out,
+                                                           int B, int H, int W, int C, int COUT, int R, int S,
+                                                           int stride, int pad, int Ho, int Wo, int bits,
+                                                           int zero_point, int T, int rowlen, int patch_bytes) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int K = R * S * C, KP = T * 32;
+  int8_t *wl = reinterpret_cast<int8_t *>(lds);                          // [64][KP]
+  uint16_t *tab = reinterpret_cast<uint16_t *>(lds + 64 * KP);           // [KP]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 31, g = lane >> 5;
+  int8_t *patch = reinterpret_cast<int8_t *>(lds + 64 * KP + 2 * KP) + wave * patch_bytes;
+  const int co0 = blockIdx.y * 64;
+
+  for (int i = tid; i < 64 * KP; i += 256) {
+    const int co = co0 + i / KP, k = i % KP;
+    wl[i] = (co < COUT && k < K) ? Wt[(long long)co * K + k] : (int8_t)0;
+  }
+  for (int k = tid; k < KP; k += 256) tab[k] = k < K ? (uint16_t)((k / (S * C)) * rowlen + (k % (S * C))) : (uint16_t)0xFFFF;
+
+  const int gpr = (Wo + 31) / 32;
+  const long long group = (long long)blockIdx.x * 4 + wave;
+  const bool active = group < (long long)B * Ho * gpr;
+  const int gx = (int)(group % gpr);
+  const int oy = (int)((group / gpr) % Ho);
+  const int b = (int)(group / ((long long)gpr * Ho));
+  const int ox0 = gx * 32;
+  if (active) {
+    for (int idx = lane; idx < R * rowlen; idx += 64) {
+      const int r = idx / rowlen, j = idx % rowlen;
+      const int iy = oy * stride + r - pad;
+      const int ix = ox0 * stride - pad + j / C;
+      int v = 0;
+      if (iy >= 0 && iy < H && ix >= 0 && ix < W) {
+        const int8_t raw = X[(((long long)b * H + iy) * W + ix) * C + (j % C)];
+        v = zero_point ? (int)(uint8_t)raw - zero_point : (int)raw;
+      }
+      patch[idx] = (int8_t)v;
+    }
+  }
+  __syncthreads();
+  if (!active) return;
+
+  v16i_t acc[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nb][r] = 0;
+  const int pix_off = li * stride * C;  // this lane's pixel inside the patch row
+  for (int t = 0; t < T; ++t) {
+    const int kb = t * 32 + g * 16;
+    uint32_t a[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        const uint32_t off = tab[kb + q * 4 + bb];
+        const uint32_t byte = off == 0xFFFFu ? 0u : (uint32_t)(uint8_t)patch[off + pix_off];
+        word |= byte << (8 * bb);
+      }
+      a[q] = word;
+    }
+    const v4i_t af = {(int)a[0], (int)a[1], (int)a[2], (int)a[3]};
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KP + kb);
+      acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[nb], 0, 0, 0);
+    }
+  }
+  const int nt = (1 << bits) - 1;
+  const long long row0 = ((long long)b * Ho + oy) * Wo;
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int co = co0 + nb * 32 + li;
+    if (co >= COUT) continue;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int ox = ox0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      if (ox >= Wo) continue;
+      const long long o = (row0 + ox) * COUT + co;
+      const int v = acc[nb][r];
+      if (acc_out != nullptr) acc_out[o] = v;
+      if (codes != nullptr) {
+        int code = 0;
+        for (int k = 0; k < nt; ++k) code += v >= thr[co * nt + k] ? 1 : 0;
+        codes[o] = (uint8_t)code;
+      }
+    }
+  }
+}
+
 // ---- max-pool on codes + bit-plane packing ---------------------------------------------------------
 // codes: [B][H][W][C] uint8 -> planes [bits][B*Ho*Wo][cpad/32], window win x win, stride, pad
 // (out-of-image taps ignored).  One wave per (pixel, 64-channel group).
@@ -155,6 +257,18 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
                              int zero_point, hipStream_t s) {
   const int Ho = (H + 2 * pad - R) / stride + 1, Wo = (W + 2 * pad - S) / stride + 1;
   const long long npix = (long long)B * Ho * Wo;
+  // matrix-core kernel whenever its LDS footprint (filter block, k table, 4 patches) fits
+  const int T = (R * S * C + 31) / 32;
+  const int rowlen = (31 * stride + S) * C;
+  const int patch_bytes = (R * rowlen + 15) / 16 * 16;
+  const size_t mfma_lds = (size_t)64 * T * 32 + 2 * T * 32 + 4 * (size_t)patch_bytes;
+  if (mfma_lds <= 64 * 1024 && R * rowlen < 0xFFFF) {
+    const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
+    dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
+    hipLaunchKernelGGL(conv_i8_mfma_kernel, grid, dim3(256), mfma_lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT,
+                       R, S, stride, pad, Ho, Wo, bits, zero_point, T, rowlen, patch_bytes);
+    return hipGetLastError();
+  }
   const size_t lds = (size_t)64 * R * S * C;
   dim3 grid((unsigned)((npix + 63) / 64), (unsigned)((COUT + 63) / 64));
   hipLaunchKernelGGL(conv_i8_bn_kernel<64>, grid, dim3(256), lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT, R,

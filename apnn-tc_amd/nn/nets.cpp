@@ -1,5 +1,6 @@
 // Network builders (the counterparts of the reference's demo drivers) and the C ABI of
 // libapnn_nn.so.  See include/apnn_nn.h.
+#include <chrono>
 #include <cmath>
 #include <new>
 
@@ -146,6 +147,37 @@ int apnn_net_layer(const apnn_net *net, int index, apnn_layer_desc *out) {
   if (index < 0 || index >= (int)net->impl->layers.size()) return APNN_EINVAL;
   net->impl->layers[index]->describe(out);
   return APNN_OK;
+}
+
+int apnn_net_bench(apnn_net *net, const uint8_t *images, float *logits, int warmup, int iters, int use_graph,
+                   apnn_stream_t s, float *event_ms, double *wall_ms) {
+  if (net == nullptr || event_ms == nullptr || wall_ms == nullptr) return APNN_ENULL;
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  auto step = [&]() {
+    return use_graph ? net->impl->forward_graph(images, logits, stream) : net->impl->forward(images, logits, stream);
+  };
+  int rc = 0;
+  for (int i = 0; i < warmup && rc == 0; ++i) rc = step();
+  if (rc != 0) return rc;
+  hipError_t e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) return (int)e;
+  hipEvent_t e0, e1;
+  if ((e = hipEventCreate(&e0)) != hipSuccess) return (int)e;
+  if ((e = hipEventCreate(&e1)) != hipSuccess) return (int)e;
+  const auto t0 = std::chrono::steady_clock::now();
+  (void)hipEventRecord(e0, stream);
+  for (int i = 0; i < iters && rc == 0; ++i) rc = step();
+  (void)hipEventRecord(e1, stream);
+  e = hipStreamSynchronize(stream);
+  const auto t1 = std::chrono::steady_clock::now();
+  if (rc == 0 && e != hipSuccess) rc = (int)e;
+  if (rc == 0) {
+    (void)hipEventElapsedTime(event_ms, e0, e1);
+    *wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return rc;
 }
 
 int apnn_nn_download(void *host_dst, const void *dev_src, unsigned long long bytes) {

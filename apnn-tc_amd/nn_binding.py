@@ -11,7 +11,7 @@ NN_LIB_PATH = os.path.join(binding.PKG_DIR, "lib", "libapnn_nn.so")
 NET_ALEXNET, NET_RESNET18 = 0, 1
 LAYER_INCONV_I8, LAYER_CONV, LAYER_FC, LAYER_OUT_I8 = 0, 1, 2, 3
 NN_DECLARED_SYMBOLS = ["apnn_net_create", "apnn_net_destroy", "apnn_net_forward", "apnn_net_forward_graph",
-                       "apnn_net_layer_count", "apnn_net_layer", "apnn_nn_download"]
+                       "apnn_net_layer_count", "apnn_net_layer", "apnn_net_bench", "apnn_nn_download"]
 
 _ci, _vp = ctypes.c_int, ctypes.c_void_p
 
@@ -47,6 +47,9 @@ def nn_lib():
         L.apnn_net_layer_count.restype = _ci
         L.apnn_net_layer.argtypes = [_vp, _ci, ctypes.POINTER(LayerDesc)]
         L.apnn_net_layer.restype = _ci
+        L.apnn_net_bench.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _vp, ctypes.POINTER(ctypes.c_float),
+                                     ctypes.POINTER(ctypes.c_double)]
+        L.apnn_net_bench.restype = _ci
         L.apnn_nn_download.argtypes = [_vp, _vp, ctypes.c_ulonglong]
         L.apnn_nn_download.restype = _ci
         _lib = L

@@ -63,6 +63,13 @@ int apnn_net_forward_graph(apnn_net *net, const uint8_t *images, float *logits, 
 int apnn_net_layer_count(const apnn_net *net);
 int apnn_net_layer(const apnn_net *net, int index, apnn_layer_desc *out);
 
+/* Timing loop of the demo drivers (the reference wraps its layer launches in clock() calls,
+ * APNN-TC-nn/src/resnet18.cu:270-323): `warmup` untimed forwards, then `iters` back-to-back forwards
+ * with no host synchronisation in between; event_ms = HIP-event time, wall_ms = host wall clock, both
+ * for all `iters` forwards.  use_graph != 0 replays the captured HIP graph. */
+int apnn_net_bench(apnn_net *net, const uint8_t *images, float *logits, int warmup, int iters, int use_graph,
+                   apnn_stream_t s, float *event_ms, double *wall_ms);
+
 /* Blocking device-to-host copy for buffers owned by a network. */
 int apnn_nn_download(void *host_dst, const void *dev_src, unsigned long long bytes);
 
