@@ -113,24 +113,28 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   return nullptr;
 }
 
-// MFMA tile: largest shape that still yields one work-group per compute unit; narrow outputs
-// (<= 64 channels) take the 128x64 shape; otherwise the smallest.
-int choose_mfma_tile(int rowsA, int rowsB) {
+// MFMA tile: the largest shape that still gives every compute unit a work-group; narrow outputs
+// (<= 64 channels) take the 128x64 shape; when even 64x64 tiles leave most of the chip idle and the
+// reduction is long, the 32-row tiles whose four waves split K.
+int choose_mfma_tile(int rowsA, int rowsB, int KW) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
     return (long long)((rowsA + apnn::kMfmaTileA[t] - 1) / apnn::kMfmaTileA[t]) *
            ((rowsB + apnn::kMfmaTileB[t] - 1) / apnn::kMfmaTileB[t]);
   };
-  if (rowsB <= 64) return ntiles(3) >= cus ? 3 : 2;
-  for (int t = 0; t < 2; ++t)
-    if (ntiles(t) >= cus) return t;
-  return 2;
+  if (rowsB <= 64 && ntiles(3) >= cus) return 3;
+  if (rowsB > 64) {
+    for (int t = 0; t < 2; ++t)
+      if (ntiles(t) >= cus) return t;
+  }
+  if (ntiles(2) >= cus / 2 || KW < 16) return 2;
+  return ntiles(5) >= cus / 2 ? 5 : 4;
 }
 
 int pick_mfma_tile(int tile_pin, const KParams &p, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;

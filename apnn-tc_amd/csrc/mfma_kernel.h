@@ -92,20 +92,29 @@ __device__ __forceinline__ void static_for(F &&f) {
 // (row-major, so the 64 lanes walk 64 consecutive output channels).  rowsum / colsum hold the
 // activation sums for the symmetric-weight correction (rows for convolution, columns for the GEMM
 // entry points).  Called by all 64 lanes of the wave; no other wave touches this slab.
-template <int NCOLS, bool CONV>
+// With KS > 1 the KS waves of the work-group each hold a partial sum over their share of K in their
+// own slab (slab_stride words apart, sums included); every wave then finishes 1/KS of the elements,
+// adding the KS partial slabs.  `part` is this wave's index among them.
+template <int NCOLS, bool CONV, int KS>
 __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab, const int *rowsum,
-                                              const int *colsum, int rbase, int cbase, int lane) {
+                                              const int *colsum, int slab_stride, int part, int rbase, int cbase,
+                                              int lane) {
   constexpr int LDT = NCOLS + 1;
   auto value = [&](int row, int col) {
-    int v = slab[row * LDT + col];
-    if (p.sym) v = 2 * v - p.wmax * (CONV ? rowsum[row] : colsum[col]);
+    int v = 0, sx = 0;
+#pragma unroll
+    for (int w = 0; w < KS; ++w) {
+      v += slab[w * slab_stride + row * LDT + col];
+      sx += CONV ? rowsum[w * slab_stride + row] : colsum[w * slab_stride + col];
+    }
+    if (p.sym) v = 2 * v - p.wmax * sx;
     return v;
   };
   if (p.epi == APNN_EPI_INT32) {
     int *out = reinterpret_cast<int *>(p.out);
     if ((p.rowsB & 3) == 0) {
       // 4 channels per lane: a wave writes 1 KiB of contiguous output per step
-      for (int e = lane * 4; e < 32 * NCOLS; e += 256) {
+      for (int e = lane * 4 + part * 256; e < 32 * NCOLS; e += 256 * KS) {
         const int row = e / NCOLS, col = e % NCOLS;
         const int grow = rbase + row, gcol = cbase + col;
         if (grow < p.rowsA && gcol < p.rowsB) {
@@ -118,7 +127,7 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
         }
       }
     } else {
-      for (int e = lane; e < 32 * NCOLS; e += 64) {
+      for (int e = lane + part * 64; e < 32 * NCOLS; e += 64 * KS) {
         const int row = e / NCOLS, col = e % NCOLS;
         const int grow = rbase + row, gcol = cbase + col;
         if (grow < p.rowsA && gcol < p.rowsB) out[(long long)grow * p.rowsB + gcol] = value(row, col);
@@ -132,7 +141,7 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
   const int n_out = pooled ? 8 : 32;
   const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
   const int row_base = pooled ? rbase / 4 : rbase;
-  for (int e = lane; e < n_out * NCOLS; e += 64) {
+  for (int e = lane + part * 64; e < n_out * NCOLS; e += 64 * KS) {
     const int orow = e / NCOLS, col = e % NCOLS;
     const int grow = row_base + orow, gcol = cbase + col;
     const bool ok = grow < out_rows_total && gcol < p.rowsB;
@@ -166,7 +175,10 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
 
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
 __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
-  static_assert(WA * WB == 4, "four waves per work-group");
+  // four waves per work-group: WA x WB of them tile the output, the remaining factor KS splits K
+  static_assert(WA * WB == 4 || WA * WB == 1, "waves tile the output or all split K");
+  constexpr int KS = 4 / (WA * WB);
+  static_assert(KS == 1 || FA == 1, "the split-K reduction handles one 32-row slab");
   constexpr bool F4 = CORE == CORE_F4;
   constexpr int WPS = F4 ? 2 : 1;                 // packed words per row consumed by one k-step
   constexpr int DA = F4 ? (PA + 1) / 2 : 1;       // operand digits (FP4: plane pairs)
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 31, g = lane >> 5;
-  const int wa = wave / WB, wb = wave % WB;
+  const int wa = KS > 1 ? 0 : wave / WB, wb = KS > 1 ? 0 : wave % WB;
 
   const int tilesB = (p.rowsB + TB - 1) / TB;
   const int a0 = (blockIdx.x / tilesB) * TA;
@@ -395,8 +407,10 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   stage(smem);
   if (nchunks > 1) fetch(KC);
   __syncthreads();
-  read_words(smem, 0);
-  expand_all(af, bf);
+  if constexpr (KS == 1) {
+    read_words(smem, 0);
+    expand_all(af, bf);
+  }
   for (int ch = 0; ch < nchunks; ++ch) {
     const uint32_t *cur = smem + (ch & 1) * BUF_WORDS;
     uint32_t *nxt = smem + ((ch + 1) & 1) * BUF_WORDS;
@@ -404,6 +418,17 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
     if (more) {
       stage(nxt);  // every wave left this buffer before the barrier of the previous chunk
       if (ch + 2 < nchunks) fetch((ch + 2) * KC);
+    }
+    if constexpr (KS > 1) {
+      // split-K: wave w owns k-steps w, w + KS, ... of every chunk
+#pragma unroll
+      for (int ks = 0; ks < NKS / KS; ++ks) {
+        read_words(cur, wave + ks * KS);
+        expand_all(af, bf);
+        mfma_all();
+      }
+      __syncthreads();
+      continue;
     }
     auto advance = [&]() {
       FragT an[FA][DA], bn[FB][DB];
@@ -455,6 +480,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
   int *rowsum = slab + 32 * LDT;
   int *colsum = rowsum + 32;
+
   if (!CONV && g == 0) {
 #pragma unroll
     for (int y = 0; y < FB; ++y) colsum[y * 32 + li] = ssum[CONV ? 0 : y];
@@ -475,9 +501,16 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
         slab[(8 * (r >> 2) + 4 * g + (r & 3)) * LDT + y * 32 + li] = v;
       });
     });
-    // LDS operations of one wave complete in order: the reads below see the writes above, and the
-    // next slab's writes come after these reads
-    wave_epilogue<NCOLS, CONV>(p, slab, rowsum, colsum, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane);
+    if constexpr (KS > 1) {
+      // all KS partial slabs must be complete before any wave sums them
+      __syncthreads();
+      const int *base = reinterpret_cast<const int *>(smem);
+      wave_epilogue<NCOLS, CONV, KS>(p, base, base + 32 * LDT, base + 32 * LDT + 32, SLAB_WORDS, wave, a0, b0, lane);
+    } else {
+      // LDS operations of one wave complete in order: the reads below see the writes above, and the
+      // next slab's writes come after these reads
+      wave_epilogue<NCOLS, CONV, 1>(p, slab, rowsum, colsum, 0, 0, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane);
+    }
   });
 }
 
@@ -504,7 +537,8 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_COUNT = 4 };
+enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
+                MT_COUNT = 6 };
 
 template <int CORE, int PA, int PB, int VW, bool CONV>
 inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t stream) {
@@ -512,6 +546,8 @@ inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t strea
     case MT_256x256: return launch_mfma<CORE, PA, PB, 4, 4, 2, 2, VW, CONV, 1>(p, stream);
     case MT_128x128: return launch_mfma<CORE, PA, PB, 2, 2, 2, 2, VW, CONV, 2>(p, stream);
     case MT_128x64: return launch_mfma<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 2>(p, stream);
+    case MT_32x32_K4: return launch_mfma<CORE, PA, PB, 1, 1, 1, 1, VW, CONV, 2>(p, stream);
+    case MT_32x64_K4: return launch_mfma<CORE, PA, PB, 1, 2, 1, 1, VW, CONV, 2>(p, stream);
     default: return launch_mfma<CORE, PA, PB, 1, 1, 2, 2, VW, CONV, 2>(p, stream);
   }
 }
