@@ -152,6 +152,23 @@ def main():
                                "hbm_gbs": round(gemm_bytes(n, n, n, w_, a_) / (t["event_ms"] * 1e-3) / 1e9, 1),
                                "verified": t["verified"]})
         extra["shapes"] = shapes
+        # ---- second headline metric: end-to-end w1a2 ResNet18 (and the AlexNet-style net) --------
+        NL = A.nn_lib()
+        nets = {}
+        for kind, nm in ((A.NET_RESNET18, "resnet18"), (A.NET_ALEXNET, "alexnet")):
+            for batch in (8, 64):
+                net = NL.apnn_net_create(kind, batch, 1, path)
+                assert net, "network construction failed"
+                img = torch.randint(0, 256, (batch, 224, 224, 3), dtype=torch.uint8, device="cuda")
+                lg = torch.empty((batch, 1000), dtype=torch.float32, device="cuda")
+                ev, wall = ctypes.c_float(), ctypes.c_double()
+                iters = 200 if batch == 8 else 50
+                A.check(NL.apnn_net_bench(net, img.data_ptr(), lg.data_ptr(), 10, iters, 0, stream, ctypes.byref(ev),
+                                          ctypes.byref(wall)), "apnn_net_bench")
+                nets["%s_w1a2_b%d" % (nm, batch)] = {"ms_per_forward": round(wall.value / iters, 4),
+                                                     "images_per_sec": round(batch * iters / wall.value * 1e3, 1)}
+                NL.apnn_net_destroy(net)
+        extra["networks"] = nets
     result["extra"] = extra
 
     # ---- CPU baseline: the scalar oracle on the same inputs, host cores ---------------------------

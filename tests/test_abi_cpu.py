@@ -65,3 +65,27 @@ def test_descriptor_entry_points_reject_bad_arguments():
     c.R = 11
     c.pad = 0
     assert L.apnn_conv(ctypes.byref(c), None) == A.EINVAL                           # filter larger than image
+
+
+def test_nn_library_exports_every_declared_symbol():
+    L = A.nn_lib()
+    header = open(os.path.join(ROOT, "include", "apnn_nn.h")).read()
+    declared = set(re.findall(r"^(?:int|void|apnn_net \*)\s*\*?(apnn_\w+)\(", header, flags=re.M))
+    assert declared == set(A.NN_DECLARED_SYMBOLS), declared ^ set(A.NN_DECLARED_SYMBOLS)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.apnn_net_layer_count(None) == 0
+    assert L.apnn_net_forward(None, None, None, None) == A.ENULL
+    assert L.apnn_net_layer(None, 0, None) == A.ENULL
+
+
+def test_edge_layer_entry_points_reject_bad_arguments():
+    L = A.lib()
+    good = 0x1000
+    assert L.apnn_conv_i8_bn(None, good, good, good, None, 1, 8, 8, 3, 64, 7, 7, 2, 3, 2, 0, None) == A.ENULL
+    assert L.apnn_conv_i8_bn(good, good, None, good, None, 1, 8, 8, 3, 64, 7, 7, 2, 3, 2, 0, None) == A.ENULL
+    assert L.apnn_conv_i8_bn(good, good, good, good, None, 1, 8, 8, 3, 64, 7, 7, 2, 3, 9, 0, None) == A.EINVAL
+    assert L.apnn_pool_pack(good, good, 1, 8, 8, 64, 100, 2, 3, 2, 1, None) == A.EINVAL      # cpad % 32
+    assert L.apnn_pool_pack(good, good, 1, 8, 8, 64, 64, 2, 3, 2, 3, None) == A.EINVAL       # pad >= window
+    assert L.apnn_unpack_sum(good, None, 4, 1, 64, 64, 2, 0, None) == A.ENULL
+    assert L.apnn_fc_i8(good, good, good, good, good, None, 0, 10, 64, None) == A.EINVAL
