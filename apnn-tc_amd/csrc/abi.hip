@@ -113,28 +113,35 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   return nullptr;
 }
 
-// MFMA tile: the largest shape that still gives every compute unit a work-group; narrow outputs
-// (<= 64 channels) take the 128x64 shape; when even 64x64 tiles leave most of the chip idle and the
+// MFMA tile.  Large problems take the 256x128 / 128x256 shape with the longer side on the operand
+// that has fewer bit-planes (its operand expansion is the cheaper one, and it is expanded four times
+// per k-step instead of two); then 128x128, 64x64 (128x64 for <= 64 output channels) while every
+// compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, int PA, int PB) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
     return (long long)((rowsA + apnn::kMfmaTileA[t] - 1) / apnn::kMfmaTileA[t]) *
            ((rowsB + apnn::kMfmaTileB[t] - 1) / apnn::kMfmaTileB[t]);
   };
+  // fraction of the launched tile area that is real output
+  auto fill = [&](int t) {
+    return (double)rowsA * rowsB / ((double)ntiles(t) * apnn::kMfmaTileA[t] * apnn::kMfmaTileB[t]);
+  };
   if (rowsB <= 64 && ntiles(3) >= cus) return 3;
   if (rowsB > 64) {
-    for (int t = 0; t < 2; ++t)
-      if (ntiles(t) >= cus) return t;
+    const int big = PA <= PB ? 6 : 7;
+    if (ntiles(big) >= cus && fill(big) >= 0.8) return big;
+    if (ntiles(1) >= cus && fill(1) >= 0.8) return 1;
   }
   if (ntiles(2) >= cus / 2 || KW < 16) return 2;
   return ntiles(5) >= cus / 2 ? 5 : 4;
 }
 
-int pick_mfma_tile(int tile_pin, const KParams &p, int *tile) {
+int pick_mfma_tile(int tile_pin, const KParams &p, int PA, int PB, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, PA, PB);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
@@ -142,11 +149,10 @@ int pick_mfma_tile(int tile_pin, const KParams &p, int *tile) {
   return APNN_OK;
 }
 
-// AUTO: the matrix-core path pays off once every wave has full 32x32 blocks to fill and the
-// reduction is long enough to amortise the epilogue; small problems stay on the VALU path.
-bool auto_prefers_mfma(const KParams &p) {
-  return (long long)p.rowsA * p.rowsB >= 256LL * 256 && p.KW >= 8;
-}
+// AUTO: the matrix-core path pays off once there are enough 32x32 blocks to fill the chip (measured
+// cross-over: about 256x256 outputs, at any reduction length); smaller, latency-bound problems stay on
+// the VALU path, whose 16x16 tiles spread them over more compute units.
+bool auto_prefers_mfma(const KParams &p) { return (long long)p.rowsA * p.rowsB >= 256LL * 256; }
 
 valu_fn valu_gemm_fn(int wb, int xb) {
   if (wb == 1 && xb == 2) return apnn::valu_gemm_1_2_x;
@@ -192,7 +198,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
+    if ((rc = pick_mfma_tile(tile_pin, p, d->wb, d->xb, &tile))) return rc;
     return (int)fn(4, tile, p, stream);
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
@@ -251,7 +257,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, &tile))) return rc;
+    if ((rc = pick_mfma_tile(tile_pin, p, d->xb, d->wb, &tile))) return rc;
     return (int)fn(vw, tile, p, stream);
   }
   valu_fn fn = valu_conv_fn(d->xb, d->wb);

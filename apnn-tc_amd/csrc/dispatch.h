@@ -42,9 +42,9 @@ APNN_DECL_MFMA4(conv, 2, 2)
 #undef APNN_DECL_MFMA4
 
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
-constexpr int kMfmaTileCount = 6;
-constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32};
-constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64};
+constexpr int kMfmaTileCount = 8;
+constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128};
+constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256};
 
 // aux_kernels.hip
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,

@@ -514,13 +514,18 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   });
 }
 
-template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
+constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB) {
+  const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * 9 * sizeof(uint32_t);
+  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32) * sizeof(int);
+  return stage > slab ? stage : slab;
+}
+
+// OCC_WANTED work-groups per compute unit if the LDS budget (160 KiB) allows it, else one
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr int LD = 9;
-  constexpr size_t stage_bytes = 2ull * (PA * TA + PB * TB) * LD * sizeof(uint32_t);
-  constexpr size_t slab_bytes = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32) * sizeof(int);
-  constexpr size_t smem_bytes = stage_bytes > slab_bytes ? stage_bytes : slab_bytes;
+  constexpr size_t smem_bytes = mfma_smem_bytes(PA, PB, FA, FB, WA, WB);
+  constexpr int OCC = (OCC_WANTED > 1 && smem_bytes * OCC_WANTED <= 160 * 1024) ? OCC_WANTED : 1;
   static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
   auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>;
   if (smem_bytes > 64 * 1024) {
@@ -538,7 +543,7 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
 }
 
 enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
-                MT_COUNT = 6 };
+                MT_256x128 = 6, MT_128x256 = 7, MT_COUNT = 8 };
 
 template <int CORE, int PA, int PB, int VW, bool CONV>
 inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t stream) {
@@ -548,6 +553,8 @@ inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t strea
     case MT_128x64: return launch_mfma<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 2>(p, stream);
     case MT_32x32_K4: return launch_mfma<CORE, PA, PB, 1, 1, 1, 1, VW, CONV, 2>(p, stream);
     case MT_32x64_K4: return launch_mfma<CORE, PA, PB, 1, 2, 1, 1, VW, CONV, 2>(p, stream);
+    case MT_256x128: return launch_mfma<CORE, PA, PB, 4, 2, 2, 2, VW, CONV, 2>(p, stream);
+    case MT_128x256: return launch_mfma<CORE, PA, PB, 2, 4, 2, 2, VW, CONV, 2>(p, stream);
     default: return launch_mfma<CORE, PA, PB, 1, 1, 2, 2, VW, CONV, 2>(p, stream);
   }
 }

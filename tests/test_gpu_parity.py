@@ -102,7 +102,7 @@ def test_gemm_symmetric_weights(G, wb, xb, path):
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=1))
 
 
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5)])
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (2, 6), (2, 7), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5), (3, 6), (3, 7)])
 def test_gemm_bn_epilogue_with_residual(G, tile, path):
     rng = np.random.default_rng(91 + tile)
     M, N, K, wb, xb, ob = 48, 160, 256, 1, 2, 2
@@ -122,12 +122,13 @@ def test_gemm_bn_epilogue_with_residual(G, tile, path):
 
 
 @pytest.mark.parametrize("path", [2, 3])
-@pytest.mark.parametrize("tile", [4, 5])
+@pytest.mark.parametrize("tile", [4, 5, 6, 7])
 @pytest.mark.parametrize("wb,xb,sym", [(1, 2, 0), (1, 2, 1), (1, 4, 1), (2, 2, 0)])
 def test_gemm_split_k_tiles(G, wb, xb, sym, tile, path):
-    """Tiles whose four waves split the reduction (partial sums combined in LDS)."""
+    """Tiles 4, 5: the four waves split the reduction (partial sums combined in LDS); 6, 7: the
+    rectangular 256x128 / 128x256 tiles."""
     rng = np.random.default_rng(60 + tile + 10 * wb + xb)
-    M, N, K = 77, 130, 1664          # K/32 = 52 words: not a multiple of the chunk
+    M, N, K = (77, 130, 1664) if tile < 6 else (300, 289, 1664)     # K/32 = 52 words: not a multiple of the chunk
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
     got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=path, tile=tile).reshape(M, N)
@@ -214,7 +215,7 @@ def test_conv_every_tile(G, tile, path):
 
 
 @pytest.mark.parametrize("pool", [0, 1, 2])
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5)])
+@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (2, 6), (2, 7), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5), (3, 6), (3, 7)])
 def test_conv_bn_epilogue(G, pool, tile, path):
     """BN-threshold requantize to a bits (+ residual / saved accumulator when not pooling,
     + avg / max pooling), packed for the next layer."""
