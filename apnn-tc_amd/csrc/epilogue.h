@@ -33,6 +33,124 @@ __device__ __forceinline__ int packed_residual(const KParams &p, int grow, int g
   return code * p.resid_scale;
 }
 
+// Per-lane view of the quantizer of one output channel: thresholds (and flip) are fetched once,
+// not once per output row.
+struct ChannelQuant {
+  int t0, t1, t2;   // thresholds when there are at most three (out_bits <= 2)
+  bool flip;
+  bool in_regs;
+};
+
+__device__ __forceinline__ ChannelQuant load_channel_quant(const KParams &p, int gcol, bool col_ok) {
+  ChannelQuant q{0, 0, 0, false, false};
+  if (p.epi != APNN_EPI_BN || !col_ok) return q;
+  q.flip = p.flip != nullptr && p.flip[gcol] != 0;
+  const int nt = (1 << p.out_bits) - 1;
+  if (nt <= 3) {
+    const int32_t *t = p.thr + (long long)gcol * nt;
+    q.t0 = t[0];
+    q.t1 = nt > 1 ? t[1] : 0x7fffffff;
+    q.t2 = nt > 2 ? t[2] : 0x7fffffff;
+    q.in_regs = true;
+  }
+  return q;
+}
+
+__device__ __forceinline__ int quantize_with(const KParams &p, const ChannelQuant &q, int v, int gcol) {
+  if (p.epi == APNN_EPI_LOWBITS) return v & ((1 << p.out_bits) - 1);
+  if (!q.in_regs) return quantize_code(p, v, gcol);
+  if (q.flip) v = -v;
+  return (v >= q.t0 ? 1 : 0) + (v >= q.t1 ? 1 : 0) + (v >= q.t2 ? 1 : 0);
+}
+
+// Quantize-and-pack stage shared by all kernels.  `value(row, col)` returns the finished int32 sum
+// of tile row `row`, tile column `col` (from LDS).  The tile has `n_rows` rows x NCOLS columns; with
+// pooling, rows 4i..4i+3 are one 2x2 window.  Work is cut into units of 64 consecutive
+// (row, column) elements -- one ballot per output bit gives two MSB-first words -- and this wave
+// takes units part, part + nparts, ...  Units are processed four at a time: all global loads of a
+// group (shortcut words, int32 residuals) are issued before any of them is consumed, so the loop
+// pays one memory round trip per four units instead of one per unit.
+template <int NCOLS, class ValueFn>
+__device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n_rows, int rbase, int cbase,
+                                          int part, int nparts) {
+  static_assert(NCOLS == 32 || NCOLS == 64 || NCOLS == 128, "tile width");
+  constexpr int UB = 4;
+  const int lane = threadIdx.x & 63;
+  const bool pooled = p.pool != APNN_POOL_NONE;
+  const int n_out = pooled ? n_rows / 4 : n_rows;
+  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
+  const int row_base = pooled ? rbase / 4 : rbase;
+  const int w32 = p.rowsB >> 5;
+  const long long rplane = (long long)p.rowsA * w32;
+  uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+  const int nunits = n_out * NCOLS / 64;
+
+  // a lane meets at most two distinct columns (NCOLS = 128: lane and lane + 64)
+  const int col0 = lane % NCOLS;
+  const ChannelQuant q0 = load_channel_quant(p, cbase + col0, cbase + col0 < p.rowsB);
+  ChannelQuant q1 = q0;
+  if (NCOLS == 128) q1 = load_channel_quant(p, cbase + col0 + 64, cbase + col0 + 64 < p.rowsB);
+
+  for (int u0 = part; u0 < nunits; u0 += nparts * UB) {
+    int v[UB], grow[UB], gcol[UB];
+    bool ok[UB];
+    uint32_t rw[UB][8];
+    int ri[UB];
+#pragma unroll
+    for (int j = 0; j < UB; ++j) {
+      const int e = (u0 + j * nparts) * 64 + lane;
+      const int orow = e / NCOLS, col = e % NCOLS;
+      grow[j] = row_base + orow;
+      gcol[j] = cbase + col;
+      ok[j] = (u0 + j * nparts) < nunits && grow[j] < out_rows_total && gcol[j] < p.rowsB;
+      v[j] = 0;
+      ri[j] = 0;
+      if (ok[j] && !pooled) {
+        const long long o = (long long)grow[j] * p.rowsB + gcol[j];
+        if (p.resid != nullptr) ri[j] = p.resid[o];
+        if (p.resid_planes != nullptr) {
+          const long long wi = (long long)grow[j] * w32 + (gcol[j] >> 5);
+          for (int b = 0; b < p.resid_bits; ++b) rw[j][b] = p.resid_planes[b * rplane + wi];
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < UB; ++j) {
+      const int e = (u0 + j * nparts) * 64 + lane;
+      const int orow = e / NCOLS, col = e % NCOLS;
+      const ChannelQuant &q = (NCOLS == 128 && col >= 64) ? q1 : q0;
+      int code = 0;
+      if (ok[j]) {
+        if (!pooled) {
+          int t = value(orow, col) + ri[j];
+          if (p.resid_planes != nullptr) {
+            const int sh = 31 - (gcol[j] & 31);
+            int rc = 0;
+            for (int b = 0; b < p.resid_bits; ++b) rc |= (int)((rw[j][b] >> sh) & 1u) << b;
+            t += rc * p.resid_scale;
+          }
+          if (p.save_acc != nullptr) p.save_acc[(long long)grow[j] * p.rowsB + gcol[j]] = t;
+          code = quantize_with(p, q, t, gcol[j]);
+        } else {
+          const int t0 = value(4 * orow, col), t1 = value(4 * orow + 1, col);
+          const int t2 = value(4 * orow + 2, col), t3 = value(4 * orow + 3, col);
+          if (p.pool == APNN_POOL_AVG2X2) {
+            code = quantize_with(p, q, (t0 + t1 + t2 + t3) / 4, gcol[j]);
+          } else {
+            code = max(max(quantize_with(p, q, t0, gcol[j]), quantize_with(p, q, t1, gcol[j])),
+                       max(quantize_with(p, q, t2, gcol[j]), quantize_with(p, q, t3, gcol[j])));
+          }
+        }
+      }
+      for (int b = 0; b < p.out_bits; ++b) {
+        const unsigned long long mask = __ballot(ok[j] && ((code >> b) & 1));
+        const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
+        if (ok[j] && (lane & 31) == 0) out[b * p.out_plane + (long long)grow[j] * w32 + (gcol[j] >> 5)] = word;
+      }
+    }
+  }
+}
+
 // tile: LDS, [TA][TB + 1] int32, row r of the tile is output row a0 + r (or, in pool order, rows
 // 4i..4i+3 are the 2x2 window a0/4 + i).  Must be called by every thread of the block after a
 // __syncthreads() that made the tile visible.
@@ -40,52 +158,8 @@ template <int TA, int TB>
 __device__ __forceinline__ void epilogue_packed(const KParams &p, const int *tile, int a0, int b0) {
   static_assert(TB % 32 == 0, "packed epilogue needs whole 32-channel words per tile row");
   constexpr int LDT = TB + 1;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nwaves = blockDim.x >> 6;
-  const bool pooled = p.pool != APNN_POOL_NONE;
-  const int n_out = pooled ? TA / 4 : TA;
-  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
-  const int row_base = pooled ? a0 / 4 : a0;
-  const int w32 = p.rowsB >> 5;
-  uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-
-  for (int unit = wave; unit < n_out * TB / 64; unit += nwaves) {
-    const int e = unit * 64 + lane;
-    const int orow = e / TB;
-    const int col = e % TB;
-    const int grow = row_base + orow;
-    const int gcol = b0 + col;
-    const bool valid = grow < out_rows_total && gcol < p.rowsB;
-    int code = 0;
-    if (valid) {
-      if (!pooled) {
-        int v = tile[orow * LDT + col];
-        const long long o = (long long)grow * p.rowsB + gcol;
-        if (p.resid != nullptr) v += p.resid[o];
-        if (p.resid_planes != nullptr) v += packed_residual(p, grow, gcol);
-        if (p.save_acc != nullptr) p.save_acc[o] = v;
-        code = quantize_code(p, v, gcol);
-      } else {
-        const int t0 = tile[(4 * orow + 0) * LDT + col];
-        const int t1 = tile[(4 * orow + 1) * LDT + col];
-        const int t2 = tile[(4 * orow + 2) * LDT + col];
-        const int t3 = tile[(4 * orow + 3) * LDT + col];
-        if (p.pool == APNN_POOL_AVG2X2) {
-          code = quantize_code(p, (t0 + t1 + t2 + t3) / 4, gcol);
-        } else {
-          const int c0 = quantize_code(p, t0, gcol), c1 = quantize_code(p, t1, gcol);
-          const int c2 = quantize_code(p, t2, gcol), c3 = quantize_code(p, t3, gcol);
-          code = max(max(c0, c1), max(c2, c3));
-        }
-      }
-    }
-    for (int b = 0; b < p.out_bits; ++b) {
-      const unsigned long long mask = __ballot(valid && ((code >> b) & 1));
-      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
-      if (valid && (lane & 31) == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
-    }
-  }
+  pack_rows<TB>(p, [&](int row, int col) { return tile[row * LDT + col]; }, TA, a0, b0, threadIdx.x >> 6,
+                blockDim.x >> 6);
 }
 
 }  // namespace apnn

@@ -135,42 +135,7 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
     }
     return;
   }
-  uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-  const int w32 = p.rowsB >> 5;
-  const bool pooled = p.pool != APNN_POOL_NONE;
-  const int n_out = pooled ? 8 : 32;
-  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
-  const int row_base = pooled ? rbase / 4 : rbase;
-  for (int e = lane + part * 64; e < n_out * NCOLS; e += 64 * KS) {
-    const int orow = e / NCOLS, col = e % NCOLS;
-    const int grow = row_base + orow, gcol = cbase + col;
-    const bool ok = grow < out_rows_total && gcol < p.rowsB;
-    int code = 0;
-    if (ok) {
-      if (!pooled) {
-        int v = value(orow, col);
-        const long long o = (long long)grow * p.rowsB + gcol;
-        if (p.resid != nullptr) v += p.resid[o];
-        if (p.resid_planes != nullptr) v += packed_residual(p, grow, gcol);
-        if (p.save_acc != nullptr) p.save_acc[o] = v;
-        code = quantize_code(p, v, gcol);
-      } else {
-        const int t0 = value(4 * orow, col), t1 = value(4 * orow + 1, col);
-        const int t2 = value(4 * orow + 2, col), t3 = value(4 * orow + 3, col);
-        if (p.pool == APNN_POOL_AVG2X2) {
-          code = quantize_code(p, (t0 + t1 + t2 + t3) / 4, gcol);
-        } else {
-          code = max(max(quantize_code(p, t0, gcol), quantize_code(p, t1, gcol)),
-                     max(quantize_code(p, t2, gcol), quantize_code(p, t3, gcol)));
-        }
-      }
-    }
-    for (int b = 0; b < p.out_bits; ++b) {
-      const unsigned long long mask = __ballot(ok && ((code >> b) & 1));
-      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
-      if (ok && (lane & 31) == 0) out[b * p.out_plane + (long long)grow * w32 + (gcol >> 5)] = word;
-    }
-  }
+  pack_rows<NCOLS>(p, value, 32, rbase, cbase, part, KS);
 }
 
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
