@@ -105,20 +105,24 @@ valu_fn mfma_gemm_fn(int wb, int xb, bool i8) {
   return nullptr;
 }
 
+// the int8 core is built for the GEMM entry points only
 valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
-  if (xb == 2 && wb == 1) return i8 ? apnn::mfma_conv_2_1_x : apnn::mfma4_conv_2_1_x;
-  if (xb == 3 && wb == 1) return i8 ? apnn::mfma_conv_3_1_x : apnn::mfma4_conv_3_1_x;
-  if (xb == 4 && wb == 1) return i8 ? apnn::mfma_conv_4_1_x : apnn::mfma4_conv_4_1_x;
-  if (xb == 2 && wb == 2) return i8 ? apnn::mfma_conv_2_2_x : apnn::mfma4_conv_2_2_x;
+  if (i8) return nullptr;
+  if (xb == 2 && wb == 1) return apnn::mfma4_conv_2_1_x;
+  if (xb == 3 && wb == 1) return apnn::mfma4_conv_3_1_x;
+  if (xb == 4 && wb == 1) return apnn::mfma4_conv_4_1_x;
+  if (xb == 2 && wb == 2) return apnn::mfma4_conv_2_2_x;
   return nullptr;
 }
 
-// MFMA tile.  Large problems take the 256x128 / 128x256 shape with the longer side on the operand
-// that has fewer bit-planes (its operand expansion is the cheaper one, and it is expanded four times
-// per k-step instead of two); then 128x128, 64x64 (128x64 for <= 64 output channels) while every
+int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTED : (int)e; }
+
+// MFMA tile.  Large problems take the 256x128 (GEMM entry points) / 128x256 (convolution) shape: the
+// longer side is on the weight operand, which has fewer bit-planes, so the cheaper operand expansion
+// is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, int PA, int PB) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
@@ -129,9 +133,14 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, int PA, int PB) {
   auto fill = [&](int t) {
     return (double)rowsA * rowsB / ((double)ntiles(t) * apnn::kMfmaTileA[t] * apnn::kMfmaTileB[t]);
   };
+  if (i8) {  // int8 core: 256x128, 128x128 and 64x64 are built
+    if (ntiles(6) >= cus && fill(6) >= 0.8) return 6;
+    return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
+  }
+  if (conv && vw == 1) return (ntiles(2) >= cus / 2 || KW < 16) ? 2 : 4;  // 32-bit loads: two tiles built
   if (rowsB <= 64 && ntiles(3) >= cus) return 3;
   if (rowsB > 64) {
-    const int big = PA <= PB ? 6 : 7;
+    const int big = conv ? 7 : 6;
     if (ntiles(big) >= cus && fill(big) >= 0.8) return big;
     if (ntiles(1) >= cus && fill(1) >= 0.8) return 1;
   }
@@ -139,9 +148,9 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, int PA, int PB) {
   return ntiles(5) >= cus / 2 ? 5 : 4;
 }
 
-int pick_mfma_tile(int tile_pin, const KParams &p, int PA, int PB, int *tile) {
+int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, PA, PB);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
@@ -198,8 +207,8 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, d->wb, d->xb, &tile))) return rc;
-    return (int)fn(4, tile, p, stream);
+    if ((rc = pick_mfma_tile(tile_pin, p, false, 4, path == APNN_PATH_MFMA_I8, &tile))) return rc;
+    return from_hip(fn(4, tile, p, stream));
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
@@ -257,8 +266,8 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, d->xb, d->wb, &tile))) return rc;
-    return (int)fn(vw, tile, p, stream);
+    if ((rc = pick_mfma_tile(tile_pin, p, true, vw, false, &tile))) return rc;
+    return from_hip(fn(vw, tile, p, stream));
   }
   valu_fn fn = valu_conv_fn(d->xb, d->wb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;

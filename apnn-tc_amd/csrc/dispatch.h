@@ -26,10 +26,6 @@ APNN_DECL_MFMA(gemm, 1, 2)
 APNN_DECL_MFMA(gemm, 1, 3)
 APNN_DECL_MFMA(gemm, 1, 4)
 APNN_DECL_MFMA(gemm, 2, 2)
-APNN_DECL_MFMA(conv, 2, 1)
-APNN_DECL_MFMA(conv, 3, 1)
-APNN_DECL_MFMA(conv, 4, 1)
-APNN_DECL_MFMA(conv, 2, 2)
 APNN_DECL_MFMA4(gemm, 1, 2)
 APNN_DECL_MFMA4(gemm, 1, 3)
 APNN_DECL_MFMA4(gemm, 1, 4)

@@ -7,6 +7,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../include/apnn_tc.h"
 #include "kparams.h"
 
@@ -70,9 +72,52 @@ __device__ __forceinline__ int quantize_with(const KParams &p, const ChannelQuan
 // takes units part, part + nparts, ...  Units are processed four at a time: all global loads of a
 // group (shortcut words, int32 residuals) are issued before any of them is consumed, so the loop
 // pays one memory round trip per four units instead of one per unit.
+//
+// q0 / q1: quantizers of the (at most two) columns this lane meets, from load_tile_quant().
+// res_lds: when not null, the shortcut words of the tile, [resid_bits][n_rows][NCOLS/32], already in
+// LDS (fetched by the kernel before its K loop, so their latency is hidden); otherwise shortcut words
+// are read from global memory inside the loop.
+template <int NCOLS>
+__device__ __forceinline__ void load_tile_quant(const KParams &p, int cbase, ChannelQuant &q0, ChannelQuant &q1) {
+  const int col0 = (threadIdx.x & 63) % NCOLS;
+  q0 = load_channel_quant(p, cbase + col0, cbase + col0 < p.rowsB);
+  q1 = q0;
+  if (NCOLS == 128) q1 = load_channel_quant(p, cbase + col0 + 64, cbase + col0 + 64 < p.rowsB);
+}
+
+// Shortcut words of a tile of n_rows x NCOLS outputs, two planes at most: word i of the tile is
+// (plane b, row r, column word c) with i = (b * n_rows + r) * (NCOLS/32) + c.  prefetch: thread
+// `t` of `nthreads` keeps words t, t + nthreads, ... in registers; publish: writes them to LDS.
+template <int NCOLS, int NREGS>
+__device__ __forceinline__ void shortcut_prefetch(const KParams &p, int n_rows, int rbase, int cbase, int t,
+                                                  int nthreads, uint32_t (&regs)[NREGS]) {
+  constexpr int CW = NCOLS / 32;
+  const int w32 = p.rowsB >> 5;
+  const long long rplane = (long long)p.rowsA * w32;
+  const int total = p.resid_bits * n_rows * CW;
+#pragma unroll
+  for (int j = 0; j < NREGS; ++j) {
+    const int i = t + j * nthreads;
+    uint32_t w = 0;
+    if (i < total) {
+      const int c = i % CW, r = (i / CW) % n_rows, b = i / (CW * n_rows);
+      const int grow = rbase + r, gw = (cbase >> 5) + c;
+      if (grow < p.rowsA && gw < w32) w = p.resid_planes[b * rplane + (long long)grow * w32 + gw];
+    }
+    regs[j] = w;
+  }
+}
+
+template <int NREGS>
+__device__ __forceinline__ void shortcut_publish(uint32_t *res_lds, int t, int nthreads, const uint32_t (&regs)[NREGS]) {
+#pragma unroll
+  for (int j = 0; j < NREGS; ++j) res_lds[t + j * nthreads] = regs[j];
+}
+
 template <int NCOLS, class ValueFn>
 __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n_rows, int rbase, int cbase,
-                                          int part, int nparts) {
+                                          int part, int nparts, const ChannelQuant &q0, const ChannelQuant &q1,
+                                          const uint32_t *res_lds) {
   static_assert(NCOLS == 32 || NCOLS == 64 || NCOLS == 128, "tile width");
   constexpr int UB = 4;
   const int lane = threadIdx.x & 63;
@@ -85,11 +130,8 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
   uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
   const int nunits = n_out * NCOLS / 64;
 
-  // a lane meets at most two distinct columns (NCOLS = 128: lane and lane + 64)
-  const int col0 = lane % NCOLS;
-  const ChannelQuant q0 = load_channel_quant(p, cbase + col0, cbase + col0 < p.rowsB);
-  ChannelQuant q1 = q0;
-  if (NCOLS == 128) q1 = load_channel_quant(p, cbase + col0 + 64, cbase + col0 + 64 < p.rowsB);
+  const bool res_global = p.resid_planes != nullptr && res_lds == nullptr;
+  const bool res_local = p.resid_planes != nullptr && res_lds != nullptr;
 
   for (int u0 = part; u0 < nunits; u0 += nparts * UB) {
     int v[UB], grow[UB], gcol[UB];
@@ -108,7 +150,7 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
       if (ok[j] && !pooled) {
         const long long o = (long long)grow[j] * p.rowsB + gcol[j];
         if (p.resid != nullptr) ri[j] = p.resid[o];
-        if (p.resid_planes != nullptr) {
+        if (res_global) {
           const long long wi = (long long)grow[j] * w32 + (gcol[j] >> 5);
           for (int b = 0; b < p.resid_bits; ++b) rw[j][b] = p.resid_planes[b * rplane + wi];
         }
@@ -123,10 +165,13 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
       if (ok[j]) {
         if (!pooled) {
           int t = value(orow, col) + ri[j];
-          if (p.resid_planes != nullptr) {
+          if (res_global || res_local) {
             const int sh = 31 - (gcol[j] & 31);
             int rc = 0;
-            for (int b = 0; b < p.resid_bits; ++b) rc |= (int)((rw[j][b] >> sh) & 1u) << b;
+            for (int b = 0; b < p.resid_bits; ++b) {
+              const uint32_t w = res_local ? res_lds[(b * n_rows + orow) * (NCOLS / 32) + (col >> 5)] : rw[j][b];
+              rc |= (int)((w >> sh) & 1u) << b;
+            }
             t += rc * p.resid_scale;
           }
           if (p.save_acc != nullptr) p.save_acc[(long long)grow[j] * p.rowsB + gcol[j]] = t;
@@ -151,15 +196,136 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
   }
 }
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for_e(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for_e<I + 1, N>(f);
+  }
+}
+
+// Burst version of pack_rows for the common case (at most two output bits, no int32 residual, no
+// saved accumulator, shortcut words -- if any -- already in LDS).  Units are handled eight at a time
+// with compile-time indices inside a group: the eight LDS gathers are issued back to back, the codes
+// are computed in registers, and each packed word is parked in the lane whose index equals its
+// output row; after the last group every lane stores its own row's words, one plane at a time.
+// NR = tile rows, NPARTS waves share the tile (unit = u * NPARTS + part).
+template <int NR, int NCOLS, int NPARTS, class ValueFn>
+__device__ __forceinline__ void pack_rows_burst(const KParams &p, ValueFn value, int rbase, int cbase, int part,
+                                                const ChannelQuant &q0, const ChannelQuant &q1,
+                                                const uint32_t *res_lds) {
+  static_assert(NCOLS == 32 || NCOLS == 64 || NCOLS == 128, "tile width");
+  constexpr int CW = NCOLS / 32;
+  constexpr int G = 8;
+  const int lane = threadIdx.x & 63;
+  const bool pooled = p.pool != APNN_POOL_NONE;
+  const int n_out = pooled ? NR / 4 : NR;
+  const int total = n_out * NCOLS / 64;  // units in the tile
+  const int out_rows_total = pooled ? p.rowsA / 4 : p.rowsA;
+  const int row_base = pooled ? rbase / 4 : rbase;
+  const int w32 = p.rowsB >> 5;
+  const bool shortcut = p.resid_planes != nullptr;
+  uint32_t mine[2][CW];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int c = 0; c < CW; ++c) mine[b][c] = 0;
+
+#pragma unroll 1
+  for (int u0 = 0; u0 * NPARTS < total; u0 += G) {
+    int code[G];
+    static_for_e<0, G>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const int unit = (u0 + j) * NPARTS + part;
+      const int e = unit * 64 + lane;
+      const int orow = e / NCOLS, col = e % NCOLS;
+      const int gcol = cbase + col;
+      const ChannelQuant &q = (NCOLS == 128 && col >= 64) ? q1 : q0;
+      int c = 0;
+      if (unit < total) {
+        if (!pooled) {
+          int t = value(orow, col);
+          if (shortcut) {
+            const int sh = 31 - (gcol & 31);
+            int rc = 0;
+            for (int b = 0; b < p.resid_bits; ++b)
+              rc |= (int)((res_lds[(b * NR + orow) * CW + (col >> 5)] >> sh) & 1u) << b;
+            t += rc * p.resid_scale;
+          }
+          c = quantize_with(p, q, t, gcol);
+        } else {
+          const int t0 = value(4 * orow, col), t1 = value(4 * orow + 1, col);
+          const int t2 = value(4 * orow + 2, col), t3 = value(4 * orow + 3, col);
+          if (p.pool == APNN_POOL_AVG2X2) {
+            c = quantize_with(p, q, (t0 + t1 + t2 + t3) / 4, gcol);
+          } else {
+            c = max(max(quantize_with(p, q, t0, gcol), quantize_with(p, q, t1, gcol)),
+                    max(quantize_with(p, q, t2, gcol), quantize_with(p, q, t3, gcol)));
+          }
+        }
+      }
+      code[j] = c;
+    });
+    static_for_e<0, G>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      const int unit = (u0 + j) * NPARTS + part;  // out-of-range units have code 0 and match no lane below
+      static_for_e<0, 2>([&](auto bc) {
+        constexpr int b = decltype(bc)::value;
+        const unsigned long long mask = __ballot((code[j] >> b) & 1);
+        const uint32_t lo = __brev((uint32_t)mask), hi = __brev((uint32_t)(mask >> 32));
+        // tile word index 2*unit + h  ->  row (2*unit + h) / CW, column word (2*unit + h) % CW
+        if constexpr (CW == 1) {
+          if (lane == 2 * unit) mine[b][0] = lo;
+          if (lane == 2 * unit + 1) mine[b][0] = hi;
+        } else if constexpr (CW == 2) {
+          if (lane == unit) {
+            mine[b][0] = lo;
+            mine[b][1] = hi;
+          }
+        } else {
+          if (lane == (unit >> 1)) {
+            if (unit & 1) {
+              mine[b][2] = lo;
+              mine[b][3] = hi;
+            } else {
+              mine[b][0] = lo;
+              mine[b][1] = hi;
+            }
+          }
+        }
+      });
+    });
+  }
+  // lane r owns output row r of the tile, if that row belongs to one of this wave's units
+  const int owner_unit = CW == 1 ? (lane >> 1) : CW == 2 ? lane : 2 * lane;
+  const int grow = row_base + lane;
+  if (lane < n_out && grow < out_rows_total && (owner_unit % NPARTS) == (NPARTS == 1 ? 0 : part)) {
+    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+    for (int b = 0; b < p.out_bits; ++b) {
+      uint32_t *dst = out + b * p.out_plane + (long long)grow * w32 + (cbase >> 5);
+#pragma unroll
+      for (int c = 0; c < CW; ++c)
+        if ((cbase >> 5) + c < w32) dst[c] = b == 0 ? mine[0][c] : mine[1][c];
+    }
+  }
+}
+
 // tile: LDS, [TA][TB + 1] int32, row r of the tile is output row a0 + r (or, in pool order, rows
 // 4i..4i+3 are the 2x2 window a0/4 + i).  Must be called by every thread of the block after a
-// __syncthreads() that made the tile visible.
+// __syncthreads() that made the tile (and res_lds, if used) visible.
 template <int TA, int TB>
-__device__ __forceinline__ void epilogue_packed(const KParams &p, const int *tile, int a0, int b0) {
+__device__ __forceinline__ void epilogue_packed(const KParams &p, const int *tile, int a0, int b0,
+                                                const ChannelQuant &q0, const ChannelQuant &q1,
+                                                const uint32_t *res_lds) {
   static_assert(TB % 32 == 0, "packed epilogue needs whole 32-channel words per tile row");
   constexpr int LDT = TB + 1;
-  pack_rows<TB>(p, [&](int row, int col) { return tile[row * LDT + col]; }, TA, a0, b0, threadIdx.x >> 6,
-                blockDim.x >> 6);
+  auto value = [&](int row, int col) { return tile[row * LDT + col]; };
+  if (p.out_bits <= 2 && p.resid == nullptr && p.save_acc == nullptr &&
+      (p.resid_planes == nullptr || res_lds != nullptr)) {
+    pack_rows_burst<TA, TB, 4>(p, value, a0, b0, threadIdx.x >> 6, q0, q1, res_lds);
+  } else {
+    pack_rows<TB>(p, value, TA, a0, b0, threadIdx.x >> 6, blockDim.x >> 6, q0, q1, res_lds);
+  }
 }
 
 }  // namespace apnn

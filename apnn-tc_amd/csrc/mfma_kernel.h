@@ -98,7 +98,8 @@ __device__ __forceinline__ void static_for(F &&f) {
 template <int NCOLS, bool CONV, int KS>
 __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab, const int *rowsum,
                                               const int *colsum, int slab_stride, int part, int rbase, int cbase,
-                                              int lane) {
+                                              int lane, const ChannelQuant &q0, const ChannelQuant &q1,
+                                              const uint32_t *res_lds) {
   constexpr int LDT = NCOLS + 1;
   auto value = [&](int row, int col) {
     int v = 0, sx = 0;
@@ -135,7 +136,12 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
     }
     return;
   }
-  pack_rows<NCOLS>(p, value, 32, rbase, cbase, part, KS);
+  if (p.out_bits <= 2 && p.resid == nullptr && p.save_acc == nullptr &&
+      (p.resid_planes == nullptr || res_lds != nullptr)) {
+    pack_rows_burst<32, NCOLS, KS>(p, value, rbase, cbase, part, q0, q1, res_lds);
+  } else {
+    pack_rows<NCOLS>(p, value, 32, rbase, cbase, part, KS, q0, q1, res_lds);
+  }
 }
 
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
@@ -291,6 +297,22 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
   for (int pl = 0; pl < PB; ++pl) rotB[pl] = (uint32_t)(4 * g - pl) & 31u;
 
+  // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop
+  constexpr int NCOLS_E = FB * 32;
+  constexpr int RES_REGS = NCOLS_E / 32;  // two planes x 32 rows x NCOLS/32 words over 64 lanes
+  ChannelQuant q0{}, q1{};
+  uint32_t res_regs[FA][RES_REGS];
+  bool res_prefetched = false;
+  if (p.epi != APNN_EPI_INT32) {
+    load_tile_quant<NCOLS_E>(p, b0 + wb * FB * 32, q0, q1);
+    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE) {
+#pragma unroll
+      for (int x = 0; x < FA; ++x)
+        shortcut_prefetch<NCOLS_E, RES_REGS>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64, res_regs[x]);
+      res_prefetched = true;
+    }
+  }
+
   // packed words of this lane's rows for one k-step
   uint32_t wA[FA][PA], wB[FB][PB];
   auto read_words = [&](const uint32_t *buf, int ks) {
@@ -440,11 +462,13 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   // slab turns the matrix-core layout (register r of a block = row 8*(r/4) + 4*g + r%4, column li)
   // into row-major order for coalesced stores and 64-channel ballots.
   constexpr int NCOLS = FB * 32, LDT = NCOLS + 1;
-  constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS;
+  constexpr int RES_WORDS = 2 * 32 * (NCOLS / 32);
+  constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS + RES_WORDS;
   __syncthreads();  // every wave is done with the staging buffers
   int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
   int *rowsum = slab + 32 * LDT;
   int *colsum = rowsum + 32;
+  uint32_t *res_lds = reinterpret_cast<uint32_t *>(colsum + NCOLS);
 
   if (!CONV && g == 0) {
 #pragma unroll
@@ -453,6 +477,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   static_for<0, FA>([&](auto xc) {
     constexpr int x = decltype(xc)::value;
     if (CONV && g == 0) rowsum[li] = ssum[CONV ? x : 0];
+    if (res_prefetched) shortcut_publish<RES_REGS>(res_lds, lane, 64, res_regs[x]);
     static_for<0, FB>([&](auto yc) {
       constexpr int y = decltype(yc)::value;
       static_for<0, 16>([&](auto rc) {
@@ -470,18 +495,20 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
       // all KS partial slabs must be complete before any wave sums them
       __syncthreads();
       const int *base = reinterpret_cast<const int *>(smem);
-      wave_epilogue<NCOLS, CONV, KS>(p, base, base + 32 * LDT, base + 32 * LDT + 32, SLAB_WORDS, wave, a0, b0, lane);
+      wave_epilogue<NCOLS, CONV, KS>(p, base, base + 32 * LDT, base + 32 * LDT + 32, SLAB_WORDS, wave, a0, b0, lane,
+                                     q0, q1, res_prefetched ? res_lds : nullptr);
     } else {
       // LDS operations of one wave complete in order: the reads below see the writes above, and the
       // next slab's writes come after these reads
-      wave_epilogue<NCOLS, CONV, 1>(p, slab, rowsum, colsum, 0, 0, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane);
+      wave_epilogue<NCOLS, CONV, 1>(p, slab, rowsum, colsum, 0, 0, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane,
+                                    q0, q1, res_prefetched ? res_lds : nullptr);
     }
   });
 }
 
 constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB) {
   const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * 9 * sizeof(uint32_t);
-  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32) * sizeof(int);
+  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
   return stage > slab ? stage : slab;
 }
 
@@ -510,17 +537,39 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
 enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
                 MT_256x128 = 6, MT_128x256 = 7, MT_COUNT = 8 };
 
+// Which (core, family, load width, tile) combinations are built.  Every kernel instantiation costs
+// seconds of compile time, so only the shapes the dispatcher can choose are kept:
+//   int8 core : GEMM entry points only (the second matrix-core variant, for comparison runs)
+//   FP4 core  : GEMM: all but 256x256 / 128x256;  convolution: all but 256x256 / 256x128, and only
+//               the two small tiles when the stored channel count allows 32-bit loads only.
+constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile) {
+  if (core == CORE_I8) return !conv && (tile == MT_128x128 || tile == MT_64x64 || tile == MT_256x128);
+  if (!conv) return tile != MT_256x256 && tile != MT_128x256;
+  if (vw == 1) return tile == MT_64x64 || tile == MT_32x32_K4;
+  return tile != MT_256x256 && tile != MT_256x128;
+}
+
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC, int TILE>
+inline hipError_t launch_mfma_if_enabled(const KParams &p, hipStream_t stream) {
+  if constexpr (mfma_tile_enabled(CORE, CONV, VW, TILE)) {
+    return launch_mfma<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>(p, stream);
+  } else {
+    return hipErrorNotSupported;
+  }
+}
+
 template <int CORE, int PA, int PB, int VW, bool CONV>
 inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t stream) {
   switch (tile) {
-    case MT_256x256: return launch_mfma<CORE, PA, PB, 4, 4, 2, 2, VW, CONV, 1>(p, stream);
-    case MT_128x128: return launch_mfma<CORE, PA, PB, 2, 2, 2, 2, VW, CONV, 2>(p, stream);
-    case MT_128x64: return launch_mfma<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 2>(p, stream);
-    case MT_32x32_K4: return launch_mfma<CORE, PA, PB, 1, 1, 1, 1, VW, CONV, 2>(p, stream);
-    case MT_32x64_K4: return launch_mfma<CORE, PA, PB, 1, 2, 1, 1, VW, CONV, 2>(p, stream);
-    case MT_256x128: return launch_mfma<CORE, PA, PB, 4, 2, 2, 2, VW, CONV, 2>(p, stream);
-    case MT_128x256: return launch_mfma<CORE, PA, PB, 2, 4, 2, 2, VW, CONV, 2>(p, stream);
-    default: return launch_mfma<CORE, PA, PB, 1, 1, 2, 2, VW, CONV, 2>(p, stream);
+    case MT_256x256: return launch_mfma_if_enabled<CORE, PA, PB, 4, 4, 2, 2, VW, CONV, 1, MT_256x256>(p, stream);
+    case MT_128x128: return launch_mfma_if_enabled<CORE, PA, PB, 2, 2, 2, 2, VW, CONV, 2, MT_128x128>(p, stream);
+    case MT_64x64: return launch_mfma_if_enabled<CORE, PA, PB, 1, 1, 2, 2, VW, CONV, 4, MT_64x64>(p, stream);
+    case MT_128x64: return launch_mfma_if_enabled<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 4, MT_128x64>(p, stream);
+    case MT_32x32_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 1, 1, 1, VW, CONV, 4, MT_32x32_K4>(p, stream);
+    case MT_32x64_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 2, 1, 1, VW, CONV, 4, MT_32x64_K4>(p, stream);
+    case MT_256x128: return launch_mfma_if_enabled<CORE, PA, PB, 4, 2, 2, 2, VW, CONV, 2, MT_256x128>(p, stream);
+    case MT_128x256: return launch_mfma_if_enabled<CORE, PA, PB, 2, 4, 2, 2, VW, CONV, 2, MT_128x256>(p, stream);
+    default: return hipErrorNotSupported;
   }
 }
 

@@ -59,7 +59,9 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
   constexpr int NIA = (UA + NT - 1) / NT, NIB = (UB + NT - 1) / NT;
   constexpr int NS = PA + PB - 1;
   constexpr int STAGE_WORDS = (PA * LDA + PB * LDB) * KC;
-  constexpr int TILE_WORDS = TA * (TB + 1);
+  constexpr int RES_WORDS = (TB % 32 == 0) ? 2 * TA * (TB / 32) : 0;   // two shortcut planes of the tile
+  constexpr int RES_REGS = (RES_WORDS + NT - 1) / NT > 0 ? (RES_WORDS + NT - 1) / NT : 1;
+  constexpr int TILE_WORDS = TA * (TB + 1) + RES_WORDS;
   constexpr int SMEM_WORDS = STAGE_WORDS > TILE_WORDS ? STAGE_WORDS : TILE_WORDS;
 
   __shared__ __attribute__((aligned(16))) uint32_t smem[SMEM_WORDS];
@@ -117,6 +119,20 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
   }
 
   uint32_t ra_[NIA][PA][VW], rb_[NIB][PB][VW];
+
+  // quantizer and shortcut words of this tile: requested now, consumed after the K loop
+  ChannelQuant q0{}, q1{};
+  uint32_t res_regs[RES_REGS];
+  bool res_prefetched = false;
+  if constexpr (TB % 32 == 0) {
+    if (p.epi != APNN_EPI_INT32) {
+      load_tile_quant<TB>(p, b0, q0, q1);
+      if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE) {
+        shortcut_prefetch<TB, RES_REGS>(p, TA, a0, b0, tid, NT, res_regs);
+        res_prefetched = true;
+      }
+    }
+  }
 
   auto fetch = [&](int k0) {
 #pragma unroll
@@ -268,8 +284,10 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
     for (int x = 0; x < RA; ++x)
 #pragma unroll
       for (int y = 0; y < RB; ++y) tile[(ta * RA + x) * (TB + 1) + tb * RB + y] = v[x][y];
+    uint32_t *res_lds = smem + TA * (TB + 1);
+    if (res_prefetched) shortcut_publish<RES_REGS>(res_lds, tid, NT, res_regs);
     __syncthreads();
-    epilogue_packed<TA, TB>(p, tile, a0, b0);
+    epilogue_packed<TA, TB>(p, tile, a0, b0, q0, q1, res_prefetched ? res_lds : nullptr);
   }
 }
 

@@ -89,3 +89,18 @@ def test_edge_layer_entry_points_reject_bad_arguments():
     assert L.apnn_pool_pack(good, good, 1, 8, 8, 64, 64, 2, 3, 2, 3, None) == A.EINVAL       # pad >= window
     assert L.apnn_unpack_sum(good, None, 4, 1, 64, 64, 2, 0, None) == A.ENULL
     assert L.apnn_fc_i8(good, good, good, good, good, None, 0, 10, 64, None) == A.EINVAL
+
+
+def test_combinations_that_are_not_built_are_reported():
+    """Rejected before any device call, so this runs without a GPU."""
+    L = A.lib()
+    good = 0x1000
+    c = A.ConvDesc(W=good, X=good, O=good, batch=1, H=8, Wd=8, cin_pad=128, COUT=64, R=3, S=3, stride=1, pad=1,
+                   wb=1, xb=2, path=A.PATH_MFMA_I8)
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EUNSUPPORTED          # int8 core: GEMM entry points only
+    g = A.GemmDesc(W=good, X=good, D=good, M=64, N=128, K=128, wb=1, xb=2, path=A.PATH_MFMA | (1 << 8))
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # FP4 GEMM has no 256x256 tile
+    g.wb, g.xb, g.path = 3, 5, A.PATH_AUTO
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # only w1a2 / w1a3 / w1a4 / w2a2 are built
+    g.wb, g.xb, g.path = 1, 2, A.PATH_VALU | (9 << 8)
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL                # no such tile

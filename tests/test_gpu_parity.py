@@ -50,7 +50,14 @@ def test_gemm_named_entry_golden(G, wb, xb):
     assert np.array_equal(gotp, O.lowbits_pack(_golden()["gemm_" + name], M, N, xb))
 
 
-PATHS = [1, 2, 3]   # APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8
+PATHS = [1, 2, 3]   # APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8 (GEMM entry points only)
+CONV_PATHS = [1, 2]
+# (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
+# int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128
+GEMM_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)]
+CONV_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)]
+GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
+CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
 
 
 @pytest.mark.parametrize("path", PATHS)
@@ -66,8 +73,7 @@ def test_gemm_sweep_m64(G, wb, xb, nk, path):
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, nthreads=8))
 
 
-@pytest.mark.parametrize("path", PATHS)
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("path,tile", GEMM_TILES)
 @pytest.mark.parametrize("wb,xb", COMBOS)
 def test_gemm_every_tile_ragged(G, wb, xb, tile, path):
     """Row / column counts that are not multiples of any tile, every tile shape pinned."""
@@ -102,7 +108,7 @@ def test_gemm_symmetric_weights(G, wb, xb, path):
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=1))
 
 
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (2, 6), (2, 7), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5), (3, 6), (3, 7)])
+@pytest.mark.parametrize("path,tile", GEMM_TILES_PACKED)
 def test_gemm_bn_epilogue_with_residual(G, tile, path):
     rng = np.random.default_rng(91 + tile)
     M, N, K, wb, xb, ob = 48, 160, 256, 1, 2, 2
@@ -121,12 +127,11 @@ def test_gemm_bn_epilogue_with_residual(G, tile, path):
     assert np.array_equal(G.to_host(d_save).reshape(M, N), acc + resid)
 
 
-@pytest.mark.parametrize("path", [2, 3])
-@pytest.mark.parametrize("tile", [4, 5, 6, 7])
+@pytest.mark.parametrize("path,tile", [(2, 4), (2, 5), (2, 6), (3, 6)])
 @pytest.mark.parametrize("wb,xb,sym", [(1, 2, 0), (1, 2, 1), (1, 4, 1), (2, 2, 0)])
 def test_gemm_split_k_tiles(G, wb, xb, sym, tile, path):
     """Tiles 4, 5: the four waves split the reduction (partial sums combined in LDS); 6, 7: the
-    rectangular 256x128 / 128x256 tiles."""
+    rectangular 256x128 tile."""
     rng = np.random.default_rng(60 + tile + 10 * wb + xb)
     M, N, K = (77, 130, 1664) if tile < 6 else (300, 289, 1664)     # K/32 = 52 words: not a multiple of the chunk
     W = O.random_planes(rng, wb, M, K // 32)
@@ -161,7 +166,7 @@ def test_conv_named_entry_golden(G, wb, xb):
         assert np.array_equal(G.to_host(outq, np.uint32).reshape(expect.shape), expect)
 
 
-@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("path", CONV_PATHS)
 @pytest.mark.parametrize("wb,xb", COMBOS)
 @pytest.mark.parametrize("C,batch", [(128, 1), (256, 1), (512, 1), (128, 16)])
 def test_conv3x3_16x16_sweep(G, wb, xb, C, batch, path):
@@ -186,7 +191,7 @@ GEOMS = [  # batch H W cin_pad cout R stride pad halo
 ]
 
 
-@pytest.mark.parametrize("path", PATHS)
+@pytest.mark.parametrize("path", CONV_PATHS)
 @pytest.mark.parametrize("geom", GEOMS)
 @pytest.mark.parametrize("wb,xb,sym", [(1, 2, 0), (1, 2, 1), (2, 2, 1), (1, 4, 0), (1, 3, 1)])
 def test_conv_general_geometry(G, geom, wb, xb, sym, path):
@@ -201,8 +206,7 @@ def test_conv_general_geometry(G, geom, wb, xb, sym, path):
     assert np.array_equal(got, expect)
 
 
-@pytest.mark.parametrize("path", PATHS)
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("path,tile", CONV_TILES)
 def test_conv_every_tile(G, tile, path):
     rng = np.random.default_rng(400 + tile)
     batch, H, Wd, C, cout = 2, 10, 6, 128, 72
@@ -215,7 +219,7 @@ def test_conv_every_tile(G, tile, path):
 
 
 @pytest.mark.parametrize("pool", [0, 1, 2])
-@pytest.mark.parametrize("path,tile", [(1, 0), (1, 1), (1, 2), (2, 0), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (2, 6), (2, 7), (3, 0), (3, 1), (3, 2), (3, 3), (3, 4), (3, 5), (3, 6), (3, 7)])
+@pytest.mark.parametrize("path,tile", CONV_TILES_PACKED)
 def test_conv_bn_epilogue(G, pool, tile, path):
     """BN-threshold requantize to a bits (+ residual / saved accumulator when not pooling,
     + avg / max pooling), packed for the next layer."""
@@ -375,10 +379,10 @@ def test_unpack_sum_and_fc_i8(G):
     assert np.allclose(d_out.cpu().numpy().reshape(B, N), expect, rtol=1e-6, atol=1e-6)
 
 
-@pytest.mark.parametrize("path", PATHS)
-def test_conv_packed_residual(G, path):
+@pytest.mark.parametrize("path,tile", CONV_TILES_PACKED + [(0, None)])
+def test_conv_packed_residual(G, path, tile):
     """Identity shortcut: the block input's packed codes are added, scaled, before the thresholds."""
-    rng = np.random.default_rng(970 + path)
+    rng = np.random.default_rng(970 + path + 7 * (tile or 0))
     batch, H, Wd, C, wb, xb, ob = 2, 14, 14, 128, 1, 2, 2
     X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
     Wt = O.random_planes(rng, wb, C * 9, C // 32)
@@ -389,6 +393,6 @@ def test_conv_packed_residual(G, path):
     thr = np.sort(rng.integers(-100, 100, size=(C, 3)), axis=1).astype(np.int32)
     d_thr, d_sp = G.to_dev(thr), G.to_dev(short_planes)
     epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, resid_planes=d_sp, resid_bits=2, resid_scale=24)
-    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, **kw).view(np.uint32).reshape(ob, -1, C // 32)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(ob, -1, C // 32)
     q = O.bn_quantize(acc + 24 * short.astype(np.int32), None, thr, None, ob)
     assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
