@@ -51,6 +51,7 @@ _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2",
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
 DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
                                                 "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
+                                                "apnn_conv_i8_bn_pack", "apnn_pool_planes",
                                                 "apnn_device_cus", "apnn_version"]
 
 
@@ -104,6 +105,10 @@ def lib():
         L.apnn_pack_bits.restype = _ci
         L.apnn_conv_i8_bn.argtypes = [_vp] * 5 + [_ci] * 11 + [_vp]
         L.apnn_conv_i8_bn.restype = _ci
+        L.apnn_conv_i8_bn_pack.argtypes = [_vp] * 4 + [_ci] * 11 + [_vp]
+        L.apnn_conv_i8_bn_pack.restype = _ci
+        L.apnn_pool_planes.argtypes = [_vp, _vp] + [_ci] * 8 + [_vp]
+        L.apnn_pool_planes.restype = _ci
         L.apnn_pool_pack.argtypes = [_vp, _vp] + [_ci] * 9 + [_vp]
         L.apnn_pool_pack.restype = _ci
         L.apnn_unpack_sum.argtypes = [_vp, _vp, ctypes.c_longlong] + [_ci] * 5 + [_vp]

@@ -377,8 +377,30 @@ int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds
   if (codes != nullptr && (bits < 1 || bits > 8)) return APNN_EINVAL;
   if (x_zero_point < 0 || x_zero_point > 255) return APNN_EINVAL;
   if ((long long)64 * R * S * C > 64 * 1024) return APNN_EUNSUPPORTED;  // filter block must fit in LDS
-  return (int)apnn::launch_conv_i8_bn(X, Wt, thresholds, codes, acc_out, B, H, W, C, COUT, R, S, stride, pad, bits,
-                                      x_zero_point, static_cast<hipStream_t>(s));
+  return from_hip(apnn::launch_conv_i8_bn(X, Wt, thresholds, codes, acc_out, nullptr, B, H, W, C, COUT, R, S, stride,
+                                          pad, bits, x_zero_point, static_cast<hipStream_t>(s)));
+}
+
+int apnn_conv_i8_bn_pack(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint32_t *planes, int B, int H,
+                         int W, int C, int COUT, int R, int S, int stride, int pad, int bits, int x_zero_point,
+                         apnn_stream_t s) {
+  if (X == nullptr || Wt == nullptr || thresholds == nullptr || planes == nullptr) return APNN_ENULL;
+  if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || COUT <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0)
+    return APNN_EINVAL;
+  if (H + 2 * pad < R || W + 2 * pad < S || (COUT % 32) != 0 || bits < 1 || bits > 8) return APNN_EINVAL;
+  if (x_zero_point < 0 || x_zero_point > 255) return APNN_EINVAL;
+  if (C > 4) return APNN_EUNSUPPORTED;
+  return from_hip(apnn::launch_conv_i8_bn(X, Wt, thresholds, nullptr, nullptr, planes, B, H, W, C, COUT, R, S, stride,
+                                          pad, bits, x_zero_point, static_cast<hipStream_t>(s)));
+}
+
+int apnn_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, int W, int cpad, int bits, int win, int stride,
+                     int pad, apnn_stream_t s) {
+  if (in == nullptr || out == nullptr) return APNN_ENULL;
+  if (B <= 0 || H <= 0 || W <= 0 || cpad <= 0 || (cpad % 32) != 0 || bits < 1 || bits > 8) return APNN_EINVAL;
+  if (win <= 0 || stride <= 0 || pad < 0 || pad >= win || H + 2 * pad < win || W + 2 * pad < win) return APNN_EINVAL;
+  return (int)apnn::launch_pool_planes(in, out, B, H, W, cpad / 32, bits, win, stride, pad,
+                                       static_cast<hipStream_t>(s));
 }
 
 int apnn_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits, int win,

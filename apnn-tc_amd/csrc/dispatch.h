@@ -48,8 +48,10 @@ hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, 
 
 // nn_kernels.hip
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
-                             int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
-                             int zero_point, hipStream_t s);
+                             uint32_t *planes, int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad,
+                             int bits, int zero_point, hipStream_t s);
+hipError_t launch_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, int W, int cw, int bits, int win,
+                              int stride, int pad, hipStream_t s);
 hipError_t launch_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H, int W, int C, int cpad, int bits,
                             int win, int stride, int pad, hipStream_t s);
 hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad,

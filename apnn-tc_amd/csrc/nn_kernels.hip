@@ -169,6 +169,186 @@ __global__ __launch_bounds__(256) void conv_i8_mfma_kernel(const int8_t *__restr
   }
 }
 
+// ---- int8 first convolution for C <= 4 (images), dword-per-pixel patch ------------------------------
+// Same implicit GEMM as above, but the LDS patch stores every input pixel as one dword
+// (c0, c1, c2, c3-or-zero), and K is laid out per filter row as S pixels x 4 bytes rounded up to whole
+// k-steps of 32.  A lane's 16 operand bytes of a k-step are then four consecutive, 4-byte aligned
+// dwords of the patch -- four LDS dword reads instead of thirty-two byte reads through a k table.  The
+// padding bytes of K carry zero weights, so whatever the patch holds there does not matter.
+// Output: uint8 codes, int32 sums and / or MSB-first bit-planes [bits][B*Ho*Wo][COUT/32].
+__global__ __launch_bounds__(256) void conv_i8_c4_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                         const int32_t *__restrict__ thr,
+                                                         uint8_t *__restrict__ codes, int32_t *__restrict__ acc_out,
+                                                         uint32_t *__restrict__ planes, int B, int H, int W, int C,
+                                                         int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
+                                                         int bits, int zero_point, int KR, int PW, int patch_words) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int KP = R * KR * 32;
+  const int KPL = KP + 16;  // row pitch in LDS: 16 B of padding spreads the 32 rows over the banks
+  int8_t *wl = reinterpret_cast<int8_t *>(lds);  // [64][KPL]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 31, g = lane >> 5;
+  uint32_t *patch = reinterpret_cast<uint32_t *>(lds + 64 * KPL) + wave * patch_words;  // [R][PW] pixels
+  const int co0 = blockIdx.y * 64;
+
+  for (int i = tid; i < 64 * KP; i += 256) {
+    const int co = co0 + i / KP, k = i % KP;
+    const int r = k / (KR * 32), rem = k % (KR * 32);
+    const int sx = rem >> 2, c = rem & 3;
+    wl[(i / KP) * KPL + k] =
+        (co < COUT && sx < S && c < C) ? Wt[(((long long)co * R + r) * S + sx) * C + c] : (int8_t)0;
+  }
+
+  __syncthreads();  // filter block staged once per work-group
+
+  // Each wave walks over pixel groups (32 consecutive output pixels of one output row) with a
+  // grid-wide stride; its patch is private, so no work-group barrier is needed inside the loop
+  // (LDS operations of one wave complete in order).
+  const int gpr = (Wo + 31) / 32;
+  const long long ngroups = (long long)B * Ho * gpr;
+  const int nt = (1 << bits) - 1;
+  const long long rows_total = (long long)B * Ho * Wo;
+  const int cw32 = COUT >> 5;
+  int t0[2], t1[2], t2[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int co = co0 + nb * 32 + li;
+    t0[nb] = t1[nb] = t2[nb] = 0x7fffffff;
+    if (co < COUT && thr != nullptr && nt <= 3) {
+      t0[nb] = thr[co * nt];
+      if (nt > 1) t1[nb] = thr[co * nt + 1];
+      if (nt > 2) t2[nb] = thr[co * nt + 2];
+    }
+  }
+  for (long long group = (long long)blockIdx.x * 4 + wave; group < ngroups; group += (long long)gridDim.x * 4) {
+    const int gx = (int)(group % gpr);
+    const int oy = (int)((group / gpr) % Ho);
+    const int b = (int)(group / ((long long)gpr * Ho));
+    const int ox0 = gx * 32;
+    // patch staging, eight pixels per lane at a time: all global byte loads of a batch are issued
+    // before the first one is consumed (one memory round trip per batch, not per pixel)
+    for (int base = 0; base < patch_words; base += 64 * 8) {
+      uint8_t raw[8][4];
+      bool inside[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * 64 + lane;
+        const int r = idx / PW, px = idx % PW;
+        const int iy = oy * stride + r - pad;
+        const int ix = ox0 * stride - pad + px;
+        inside[j] = idx < patch_words && r < R && iy >= 0 && iy < H && ix >= 0 && ix < W;
+        const int8_t *src = X + (((long long)b * H + (inside[j] ? iy : 0)) * W + (inside[j] ? ix : 0)) * C;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) raw[j][c] = (c < C && inside[j]) ? (uint8_t)src[c] : (uint8_t)0;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * 64 + lane;
+        uint32_t word = 0;
+        if (inside[j]) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            if (c < C) {
+              const int v = zero_point ? (int)raw[j][c] - zero_point : (int)(int8_t)raw[j][c];
+              word |= (uint32_t)(uint8_t)(int8_t)v << (8 * c);
+            }
+          }
+        }
+        if (idx < patch_words) patch[idx] = word;
+      }
+    }
+
+    v16i_t acc[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][r] = 0;
+    for (int r = 0; r < R; ++r) {
+      for (int h = 0; h < KR; ++h) {
+        const uint32_t *ap = patch + r * PW + li * stride + h * 8 + g * 4;
+        const v4i_t af = {(int)ap[0], (int)ap[1], (int)ap[2], (int)ap[3]};
+        const int kb = (r * KR + h) * 32 + g * 16;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KPL + kb);
+          acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[nb], 0, 0, 0);
+        }
+      }
+    }
+    const long long row0 = ((long long)b * Ho + oy) * Wo;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int co = co0 + nb * 32 + li;
+      const bool co_ok = co < COUT;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ox = ox0 + 8 * (r >> 2) + 4 * g + (r & 3);
+        const bool ok = co_ok && ox < Wo;
+        const long long o = (row0 + ox) * COUT + co;
+        const int v = acc[nb][r];
+        int code = 0;
+        if (ok && thr != nullptr) {
+          if (nt <= 3) {
+            code = (v >= t0[nb] ? 1 : 0) + (v >= t1[nb] ? 1 : 0) + (v >= t2[nb] ? 1 : 0);
+          } else {
+            for (int k = 0; k < nt; ++k) code += v >= thr[co * nt + k] ? 1 : 0;
+          }
+        }
+        if (ok && acc_out != nullptr) acc_out[o] = v;
+        if (ok && codes != nullptr) codes[o] = (uint8_t)code;
+        if (planes != nullptr) {
+          for (int bit = 0; bit < bits; ++bit) {
+            const unsigned long long mask = __ballot(ok && ((code >> bit) & 1));
+            const uint32_t word = g ? __brev((uint32_t)(mask >> 32)) : __brev((uint32_t)mask);
+            if (ok && li == 0) planes[bit * rows_total * cw32 + (row0 + ox) * cw32 + (co >> 5)] = word;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---- max-pool directly on bit-planes ----------------------------------------------------------------
+// in: [bits][B*H*W][cw] -> out: [bits][B*Ho*Wo][cw]; the maximum of two multi-bit codes is computed for
+// 32 channels at once with bitwise logic (compare from the top plane down).
+__global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
+                                                          int B, int H, int W, int cw, int bits, int win, int stride,
+                                                          int pad, int Ho, int Wo) {
+  const long long rows_in = (long long)B * H * W, rows_out = (long long)B * Ho * Wo;
+  const long long total = rows_out * cw;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (long long)gridDim.x * blockDim.x) {
+    const int wi = (int)(i % cw);
+    const long long row = i / cw;
+    const int ox = (int)(row % Wo), oy = (int)((row / Wo) % Ho), b = (int)(row / ((long long)Wo * Ho));
+    uint32_t m[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) m[p] = 0;
+    for (int r = 0; r < win; ++r) {
+      const int iy = oy * stride + r - pad;
+      if (iy < 0 || iy >= H) continue;
+      for (int sx = 0; sx < win; ++sx) {
+        const int ix = ox * stride + sx - pad;
+        if (ix < 0 || ix >= W) continue;
+        const long long rin = ((long long)b * H + iy) * W + ix;
+        uint32_t v[8];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) v[p] = p < bits ? in[p * rows_in * cw + rin * cw + wi] : 0u;
+        uint32_t gt = 0, lt = 0;  // per channel: m > v decided / m < v decided
+#pragma unroll
+        for (int p = 7; p >= 0; --p) {
+          const uint32_t diff = m[p] ^ v[p], open = ~(gt | lt);
+          gt |= open & diff & m[p];
+          lt |= open & diff & v[p];
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p) m[p] = (m[p] & ~lt) | (v[p] & lt);
+      }
+    }
+    for (int p = 0; p < bits; ++p) out[p * rows_out * cw + row * cw + wi] = m[p];
+  }
+}
+
 // ---- max-pool on codes + bit-plane packing ---------------------------------------------------------
 // codes: [B][H][W][C] uint8 -> planes [bits][B*Ho*Wo][cpad/32], window win x win, stride, pad
 // (out-of-image taps ignored).  One wave per (pixel, 64-channel group).
@@ -253,26 +433,60 @@ __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X
 }
 
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
-                             int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
-                             int zero_point, hipStream_t s) {
+                             uint32_t *planes, int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad,
+                             int bits, int zero_point, hipStream_t s) {
   const int Ho = (H + 2 * pad - R) / stride + 1, Wo = (W + 2 * pad - S) / stride + 1;
   const long long npix = (long long)B * Ho * Wo;
-  // matrix-core kernel whenever its LDS footprint (filter block, k table, 4 patches) fits
+  const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
+  dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
+  if (C <= 4) {
+    // dword-per-pixel patch kernel, persistent over pixel groups: the filter block is staged once
+    // per work-group
+    if (grid.x > 1024) grid.x = 1024;
+    const int KR = (S * 4 + 31) / 32;
+    const int PW = 31 * stride + KR * 8;
+    const int patch_words = (R * PW + 15) / 16 * 16;
+    const size_t lds = (size_t)64 * (R * KR * 32 + 16) + 4 * (size_t)patch_words * 4;
+    if (lds <= 160 * 1024) {
+      if (lds > 64 * 1024) {
+        static bool raised = false;
+        if (!raised) {
+          const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(conv_i8_c4_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+          if (e != hipSuccess) return e;
+          raised = true;
+        }
+      }
+      hipLaunchKernelGGL(conv_i8_c4_kernel, grid, dim3(256), lds, s, X, Wt, thr, codes, acc_out, planes, B, H, W, C,
+                         COUT, R, S, stride, pad, Ho, Wo, bits, zero_point, KR, PW, patch_words);
+      return hipGetLastError();
+    }
+  }
+  if (planes != nullptr) return hipErrorNotSupported;  // plane output is produced by the C <= 4 kernel only
+  // general C: byte-gather matrix-core kernel whenever its LDS footprint (filter block, k table, 4 patches) fits
   const int T = (R * S * C + 31) / 32;
   const int rowlen = (31 * stride + S) * C;
   const int patch_bytes = (R * rowlen + 15) / 16 * 16;
   const size_t mfma_lds = (size_t)64 * T * 32 + 2 * T * 32 + 4 * (size_t)patch_bytes;
   if (mfma_lds <= 64 * 1024 && R * rowlen < 0xFFFF) {
-    const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
-    dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
     hipLaunchKernelGGL(conv_i8_mfma_kernel, grid, dim3(256), mfma_lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT,
                        R, S, stride, pad, Ho, Wo, bits, zero_point, T, rowlen, patch_bytes);
     return hipGetLastError();
   }
   const size_t lds = (size_t)64 * R * S * C;
-  dim3 grid((unsigned)((npix + 63) / 64), (unsigned)((COUT + 63) / 64));
-  hipLaunchKernelGGL(conv_i8_bn_kernel<64>, grid, dim3(256), lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT, R,
+  dim3 grid2((unsigned)((npix + 63) / 64), (unsigned)((COUT + 63) / 64));
+  hipLaunchKernelGGL(conv_i8_bn_kernel<64>, grid2, dim3(256), lds, s, X, Wt, thr, codes, acc_out, B, H, W, C, COUT, R,
                      S, stride, pad, Ho, Wo, bits, zero_point);
+  return hipGetLastError();
+}
+
+hipError_t launch_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, int W, int cw, int bits, int win,
+                              int stride, int pad, hipStream_t s) {
+  const int Ho = (H + 2 * pad - win) / stride + 1, Wo = (W + 2 * pad - win) / stride + 1;
+  long long blocks = ((long long)B * Ho * Wo * cw + 255) / 256;
+  if (blocks > 262144) blocks = 262144;
+  hipLaunchKernelGGL(pool_planes_kernel, dim3((unsigned)blocks), dim3(256), 0, s, in, out, B, H, W, cw, bits, win,
+                     stride, pad, Ho, Wo);
   return hipGetLastError();
 }
 

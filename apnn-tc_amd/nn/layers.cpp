@@ -102,7 +102,10 @@ int InConv128LayerParam::initialize(Rng &rng, const uint8_t *images_gpu) {
   const double sigma = std::sqrt((double)filter_height * filter_width * input_channels * 5461.0 * 5376.0);
   const std::vector<int32_t> thr = random_thresholds(rng, output_channels, a_bit, 0.0, sigma);
   if (bn_gpu.upload(thr.data(), thr.size() * sizeof(int32_t)) != hipSuccess) return 1;
-  if (codes_gpu.allocate((size_t)batch * conv_height * conv_width * output_channels) != hipSuccess) return 1;
+  // un-pooled packed codes of the convolution (skipped when there is no pooling stage)
+  if (pool > 1 &&
+      codes_gpu.allocate((size_t)a_bit * batch * conv_height * conv_width * (out_cpad / 32) * 4) != hipSuccess)
+    return 1;
   if (output_gpu.allocate((size_t)a_bit * batch * output_height * output_width * (out_cpad / 32) * 4) != hipSuccess)
     return 1;
   input_gpu = images_gpu;
@@ -110,12 +113,13 @@ int InConv128LayerParam::initialize(Rng &rng, const uint8_t *images_gpu) {
 }
 
 int InConv128LayerParam::forward(hipStream_t stream) {
-  int rc = apnn_conv_i8_bn(reinterpret_cast<const int8_t *>(input_gpu), filter_gpu.as<int8_t>(), bn_gpu.as<int32_t>(),
-                           codes_gpu.as<uint8_t>(), nullptr, batch, input_height, input_width, input_channels,
-                           output_channels, filter_height, filter_width, stride, pad, a_bit, 128, stream);
-  if (rc != 0) return rc;
-  return apnn_pool_pack(codes_gpu.as<uint8_t>(), output_gpu.as<uint32_t>(), batch, conv_height, conv_width,
-                        output_channels, out_cpad, a_bit, pool, pool_stride, pool_pad, stream);
+  uint32_t *conv_out = pool > 1 ? codes_gpu.as<uint32_t>() : output_gpu.as<uint32_t>();
+  int rc = apnn_conv_i8_bn_pack(reinterpret_cast<const int8_t *>(input_gpu), filter_gpu.as<int8_t>(),
+                                bn_gpu.as<int32_t>(), conv_out, batch, input_height, input_width, input_channels,
+                                output_channels, filter_height, filter_width, stride, pad, a_bit, 128, stream);
+  if (rc != 0 || pool <= 1) return rc;
+  return apnn_pool_planes(conv_out, output_gpu.as<uint32_t>(), batch, conv_height, conv_width, out_cpad, a_bit, pool,
+                          pool_stride, pool_pad, stream);
 }
 
 void InConv128LayerParam::describe(apnn_layer_desc *d) const {

@@ -170,6 +170,18 @@ int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds
                     int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad, int bits,
                     int x_zero_point, apnn_stream_t s);
 
+/* Same convolution for image-like inputs (C <= 4), thresholds applied, result written directly as
+ * MSB-first bit-planes [bits][B*Ho*Wo][COUT/32] (COUT % 32 == 0): the first layer's activations never
+ * exist unpacked in memory. */
+int apnn_conv_i8_bn_pack(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint32_t *planes, int B, int H,
+                         int W, int C, int COUT, int R, int S, int stride, int pad, int bits, int x_zero_point,
+                         apnn_stream_t s);
+
+/* win x win max-pool of multi-bit codes directly on their bit-planes (32 channels per bitwise
+ * compare): in:[bits][B*H*W][cpad/32] -> out:[bits][B*Ho*Wo][cpad/32]; out-of-image taps are ignored. */
+int apnn_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, int W, int cpad, int bits, int win, int stride,
+                     int pad, apnn_stream_t s);
+
 /* win x win max-pool (stride, zero-free padding: out-of-image taps are ignored) over uint8 codes
  * [B][H][W][C], then bit-plane packing with the Bit_compression layout (NN/kernel.cuh:46-77):
  * planes:[bits][B*Ho*Wo][cpad/32].  win = stride = 1, pad = 0 packs without pooling. */

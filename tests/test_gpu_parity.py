@@ -396,3 +396,54 @@ def test_conv_packed_residual(G, path, tile):
     got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(ob, -1, C // 32)
     q = O.bn_quantize(acc + 24 * short.astype(np.int32), None, thr, None, ob)
     assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
+
+
+@pytest.mark.parametrize("R,stride,pad,H,cout,C", [(7, 2, 3, 40, 64, 3), (11, 4, 5, 67, 64, 3), (3, 1, 1, 9, 96, 4),
+                                                   (5, 2, 2, 33, 32, 1)])
+def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, cout, C):
+    """First layer with packed output, then max-pool on the bit-planes."""
+    rng = np.random.default_rng(990 + R)
+    B, bits = 2, 2
+    Xu = rng.integers(0, 256, size=(B, H, H + 3, C)).astype(np.uint8)
+    Wt = rng.integers(-128, 128, size=(cout, R, R, C)).astype(np.int8)
+    acc = O.conv_i8(Wt, (Xu.astype(np.int16) - 128).astype(np.int8), stride, pad)
+    Ho, Wo = acc.shape[1], acc.shape[2]
+    thr = np.sort(rng.integers(-60000, 60000, size=(cout, 3)), axis=1).astype(np.int32)
+    codes = O.bn_quantize(acc.reshape(-1, cout), None, thr, None, bits).reshape(acc.shape)
+    L = G.A.lib()
+    dX, dW, dT = torch.from_numpy(Xu).cuda(), G.to_dev(Wt), G.to_dev(thr)
+    rows = B * Ho * Wo
+    d_planes = G.dev_empty_i32(bits * rows * cout // 32, fill=-7)
+    G.A.check(L.apnn_conv_i8_bn_pack(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_planes), B, H, H + 3, C, cout, R, R,
+                                     stride, pad, bits, 128, None), "conv_i8_bn_pack")
+    expect = O.pack_bits(codes.reshape(rows, cout).astype(np.uint32), rows, cout, cout, bits)
+    assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect)
+    # the uint8-code / int32 outputs of the same kernel
+    d_codes = torch.empty(rows * cout, dtype=torch.uint8, device="cuda")
+    d_acc = G.dev_empty_i32(rows * cout, fill=-7)
+    G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, H + 3, C, cout, R, R,
+                                stride, pad, bits, 128, None), "conv_i8_bn")
+    assert np.array_equal(G.to_host(d_acc).reshape(acc.shape), acc)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_codes.cpu().numpy().reshape(acc.shape), codes.astype(np.uint8))
+    for win, st, pd in [(3, 2, 1), (2, 2, 0), (3, 1, 1)]:
+        pooled = _np_maxpool_codes(codes, win, st, pd)
+        prow = pooled.shape[0] * pooled.shape[1] * pooled.shape[2]
+        d_out = G.dev_empty_i32(bits * prow * cout // 32, fill=-7)
+        G.A.check(L.apnn_pool_planes(G.ptr(d_planes), G.ptr(d_out), B, Ho, Wo, cout, bits, win, st, pd, None), "pool_planes")
+        pexp = O.pack_bits(pooled.reshape(prow, cout).astype(np.uint32), prow, cout, cout, bits)
+        assert np.array_equal(G.to_host(d_out, np.uint32).reshape(pexp.shape), pexp)
+
+
+def test_pool_planes_wide_codes(G):
+    rng = np.random.default_rng(995)
+    B, H, W, C, bits = 2, 9, 11, 96, 5
+    codes = rng.integers(0, 2 ** bits, size=(B, H, W, C)).astype(np.int32)
+    planes = O.pack_bits(codes.reshape(-1, C).astype(np.uint32), B * H * W, C, C, bits)
+    d_in = G.to_dev(planes)
+    pooled = _np_maxpool_codes(codes, 3, 2, 1)
+    prow = pooled.shape[0] * pooled.shape[1] * pooled.shape[2]
+    d_out = G.dev_empty_i32(bits * prow * C // 32, fill=-7)
+    G.A.check(G.A.lib().apnn_pool_planes(G.ptr(d_in), G.ptr(d_out), B, H, W, C, bits, 3, 2, 1, None), "pool_planes")
+    pexp = O.pack_bits(pooled.reshape(prow, C).astype(np.uint32), prow, C, C, bits)
+    assert np.array_equal(G.to_host(d_out, np.uint32).reshape(pexp.shape), pexp)
