@@ -162,6 +162,11 @@ int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, i
 // cross-over: about 256x256 outputs, at any reduction length); smaller, latency-bound problems stay on
 // the VALU path, whose 16x16 tiles spread them over more compute units.
 bool auto_prefers_mfma(const KParams &p) { return (long long)p.rowsA * p.rowsB >= 256LL * 256; }
+// GEMM at exactly the cross-over size with a short reduction (64 x 1024 outputs over 1024 bits): both
+// paths sit on the launch floor and the VALU tile measures a few percent faster.
+bool auto_prefers_mfma_gemm(const KParams &p) {
+  return auto_prefers_mfma(p) && ((long long)p.rowsA * p.rowsB > 256LL * 256 || p.KW > 32);
+}
 
 valu_fn valu_gemm_fn(int wb, int xb) {
   if (wb == 1 && xb == 2) return apnn::valu_gemm_1_2_x;
@@ -204,7 +209,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->D, d->M);
 
   int tile;
-  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
     if ((rc = pick_mfma_tile(tile_pin, p, false, 4, path == APNN_PATH_MFMA_I8, &tile))) return rc;

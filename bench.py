@@ -25,6 +25,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
+FP4_MFMA_PEAK_TOPS = 10100.0   # MI355X dense fp4 MFMA (the matrix-core path feeds 2-bit digits as e2m1 codes)
+# HBM bytes per launch of the headline kernel from the hardware counters (FETCH_SIZE 190.07 KiB x 2.0
+# calibration, WRITE_SIZE 256 KiB x 1.0): see profiles/gemm_w1a2_m64_n1024_k1024.md
+HEADLINE_TRAFFIC_BYTES = 651407
 BASELINE_TOPS = 18.66          # reference README.md:142 (w1a2, M=64, N=K=1024, sm_86)
 
 
@@ -38,11 +42,18 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes (same as --extra none)")
+    ap.add_argument("--extra", default="all",
+                    help="comma list of secondary workloads to run after the headline: all, none, gemm_sweep, "
+                         "gemm_large, gemm8192 (w1a2 only), conv, nets, resnet18_b8, resnet18_b64, alexnet_b8, "
+                         "alexnet_b64")
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one 256 MiB device copy (known traffic) for counter calibration")
     args = ap.parse_args()
+    want = set(x for x in ("none" if args.no_extra else args.extra).split(",") if x)
+    def on(*names):
+        return "all" in want or any(n in want for n in names)
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -58,6 +69,8 @@ def main():
     L = A.lib()
     benchlib = ctypes.CDLL(os.path.join(os.path.dirname(A.LIB_PATH), "libapnn_bench.so"))
     benchlib.apnn_bench_gemm.argtypes = [ctypes.POINTER(A.GemmDesc), ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    benchlib.apnn_bench_conv.argtypes = [ctypes.POINTER(A.ConvDesc), ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                          ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     benchlib.apnn_bench_empty.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                           ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
@@ -122,7 +135,7 @@ def main():
         "config": {"workload": "apnn_gemm w1a2 M=64 N=1024 K=1024, weights 2b-1 (symmetric), int32 out",
                    "path": args.path, "verified_bit_exact": r["verified"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 6), "traffic": None,
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 6), "traffic": HEADLINE_TRAFFIC_BYTES,
                      "algorithmic_bytes": nbytes, "kernel_us": round(r["event_ms"] * 1e3, 4)},
     }
 
@@ -134,29 +147,84 @@ def main():
     extra["unsigned_reference_arithmetic"] = {"tops": round(ops / (ru["wall_ms"] * 1e-3) / 1e12, 4),
                                               "us": round(ru["wall_ms"] * 1e3, 4), "verified": ru["verified"]}
 
-    if not args.no_extra:
+    def time_conv(batch, C, w_, a_, fused, warmup, iters):
+        """3x3, stride 1, stored halo, 16x16 feature map, Cin = Cout = C (the reference's conv benchmark,
+        APNN-TC-lib/bmmaTensorCoreGemm/src/51_conv_w1a2_small.cu:478-512, with a batch dimension)."""
+        H = Wd = 16
+        rng = np.random.default_rng(0x5EED0003)
+        X = O.random_planes(rng, a_, batch * (H + 2) * (Wd + 2), C // 32)
+        # the halo ring holds zeros, as the reference's padded input does
+        Xv = X.reshape(a_, batch, H + 2, Wd + 2, C // 32)
+        Xv[:, :, 0], Xv[:, :, -1], Xv[:, :, :, 0], Xv[:, :, :, -1] = 0, 0, 0, 0
+        Wt = O.random_planes(rng, w_, C * 9, C // 32)
+        dW, dX = G.to_dev(Wt), G.to_dev(X)
+        if fused:
+            hi = 9 * C * ((1 << a_) - 1) * ((1 << w_) - 1) // 2
+            thr = np.sort(rng.integers(0, hi + 1, size=(C, (1 << a_) - 1)), axis=1).astype(np.int32)
+            dT = G.to_dev(thr)
+            out = G.dev_empty_i32(a_ * batch * H * Wd * C // 32, fill=-7)
+            E = G.epilogue(mode=A.EPI_BN, out_bits=a_, thr=dT)
+            nbytes = (a_ * batch * H * Wd * C + w_ * 9 * C * C + a_ * batch * H * Wd * C) // 8 + 4 * ((1 << a_) - 1) * C
+        else:
+            out = G.dev_empty_i32(batch * H * Wd * C, fill=-7)
+            E = G.epilogue()
+            nbytes = (a_ * batch * H * Wd * C + w_ * 9 * C * C) // 8 + 4 * batch * H * Wd * C
+        d = A.ConvDesc(W=dW.data_ptr(), X=dX.data_ptr(), O=out.data_ptr(), batch=batch, H=H, Wd=Wd, cin_pad=C, COUT=C,
+                       R=3, S=3, stride=1, pad=1, halo=1, wb=w_, xb=a_, weight_mode=A.WEIGHT_UNSIGNED, epi=E,
+                       path=path)
+        ev, wall = ctypes.c_float(), ctypes.c_double()
+        A.check(benchlib.apnn_bench_conv(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
+                                         ctypes.byref(wall)), "apnn_bench_conv")
+        torch.cuda.synchronize()
+        ok = None
+        if not fused and batch * C <= 1024:
+            got = G.to_host(out).reshape(batch, H, Wd, C)
+            ref = O.conv(Wt, X, batch=batch, H=H, W=Wd, cwords=C // 32, cout=C, R=3, S=3, stride=1, pad=1, halo=1,
+                         wb=w_, xb=a_, sym_w=0, nthreads=os.cpu_count() or 1)
+            ok = bool(np.array_equal(got, ref))
+        ops_c = 2.0 * batch * H * Wd * C * 9 * C
+        return {"us": round(ev.value / iters * 1e3, 3), "tops": round(ops_c / (ev.value / iters * 1e-3) / 1e12, 2),
+                "hbm_gbs": round(nbytes / (ev.value / iters * 1e-3) / 1e9, 1), "verified": ok}
+
+    if want != {"none"}:
         shapes = []
         for (w_, a_) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
-            for nk in (128, 512, 1024):
+            for nk in (128, 256, 384, 512, 640, 768, 896, 1024) if on("gemm_sweep") else ():
                 t = time_gemm(64, nk, nk, w_, a_, A.WEIGHT_UNSIGNED, 20, 200)
                 shapes.append({"shape": "w%da%d M=64 N=K=%d" % (w_, a_, nk),
                                "us": round(t["wall_ms"] * 1e3, 3),
                                "tops": round(2.0 * 64 * nk * nk / (t["wall_ms"] * 1e-3) / 1e12, 3),
                                "verified": t["verified"]})
-            for n in (2048, 4096, 8192):
+            large = (2048, 4096, 8192) if on("gemm_large") else ((8192,) if (w_, a_) == (1, 2) and on("gemm8192") else ())
+            for n in large:
                 iters = {2048: 20, 4096: 10, 8192: 3}[n]
                 t = time_gemm(n, n, n, w_, a_, A.WEIGHT_UNSIGNED, 2, iters, verify_rows=[0, n // 2 + 1, n - 1])
                 tt = 2.0 * n ** 3 / (t["event_ms"] * 1e-3) / 1e12
                 shapes.append({"shape": "w%da%d M=N=K=%d" % (w_, a_, n), "ms": round(t["event_ms"], 4),
                                "tops": round(tt, 2), "frac_int8_mfma_peak": round(tt / INT8_MFMA_PEAK_TOPS, 4),
+                               "frac_fp4_mfma_peak": round(tt / FP4_MFMA_PEAK_TOPS, 4),
                                "hbm_gbs": round(gemm_bytes(n, n, n, w_, a_) / (t["event_ms"] * 1e-3) / 1e9, 1),
                                "verified": t["verified"]})
-        extra["shapes"] = shapes
+        if shapes:
+            extra["shapes"] = shapes
+        if on("conv"):
+            convs = []
+            for (w_, a_) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
+                for batch in (1, 16):
+                    for C in (128, 256, 512, 1024) if (w_, a_) == (1, 2) else (512, 1024):
+                        for fused in (False, True):
+                            t = time_conv(batch, C, w_, a_, fused, 10, 200 if batch == 1 else 50)
+                            t["shape"] = "w%da%d 3x3 16x16 b%d Cin=Cout=%d %s" % (
+                                w_, a_, batch, C, "bn-quantize packed out" if fused else "int32 out")
+                            convs.append(t)
+            extra["conv"] = convs
         # ---- second headline metric: end-to-end w1a2 ResNet18 (and the AlexNet-style net) --------
-        NL = A.nn_lib()
         nets = {}
         for kind, nm in ((A.NET_RESNET18, "resnet18"), (A.NET_ALEXNET, "alexnet")):
             for batch in (8, 64):
+                if not on("nets", "%s_b%d" % (nm, batch)):
+                    continue
+                NL = A.nn_lib()
                 net = NL.apnn_net_create(kind, batch, 1, path)
                 assert net, "network construction failed"
                 img = torch.randint(0, 256, (batch, 224, 224, 3), dtype=torch.uint8, device="cuda")
@@ -168,7 +236,8 @@ def main():
                 nets["%s_w1a2_b%d" % (nm, batch)] = {"ms_per_forward": round(wall.value / iters, 4),
                                                      "images_per_sec": round(batch * iters / wall.value * 1e3, 1)}
                 NL.apnn_net_destroy(net)
-        extra["networks"] = nets
+        if nets:
+            extra["networks"] = nets
     result["extra"] = extra
 
     # ---- CPU baseline: the scalar oracle on the same inputs, host cores ---------------------------
