@@ -86,9 +86,11 @@ __device__ __forceinline__ void load_tile_quant(const KParams &p, int cbase, Cha
 }
 
 // Shortcut words of a tile of n_rows x NCOLS outputs, two planes at most: word i of the tile is
-// (plane b, row r, column word c) with i = (b * n_rows + r) * (NCOLS/32) + c.  prefetch: thread
-// `t` of `nthreads` keeps words t, t + nthreads, ... in registers; publish: writes them to LDS.
-template <int NCOLS, int NREGS>
+// (plane b, row r, column word c) with i = (b * n_rows + r) * (NCOLS/32) + c, or, with ROWFAST,
+// i = (b * (NCOLS/32) + c) * n_rows + r (four consecutive rows are then one 16-byte LDS read).
+// prefetch: thread `t` of `nthreads` keeps words t, t + nthreads, ... in registers; publish: writes
+// them to LDS.
+template <int NCOLS, int NREGS, bool ROWFAST = false>
 __device__ __forceinline__ void shortcut_prefetch(const KParams &p, int n_rows, int rbase, int cbase, int t,
                                                   int nthreads, uint32_t (&regs)[NREGS]) {
   constexpr int CW = NCOLS / 32;
@@ -100,7 +102,9 @@ __device__ __forceinline__ void shortcut_prefetch(const KParams &p, int n_rows, 
     const int i = t + j * nthreads;
     uint32_t w = 0;
     if (i < total) {
-      const int c = i % CW, r = (i / CW) % n_rows, b = i / (CW * n_rows);
+      const int c = ROWFAST ? (i / n_rows) % CW : i % CW;
+      const int r = ROWFAST ? i % n_rows : (i / CW) % n_rows;
+      const int b = i / (CW * n_rows);
       const int grow = rbase + r, gw = (cbase >> 5) + c;
       if (grow < p.rowsA && gw < w32) w = p.resid_planes[b * rplane + (long long)grow * w32 + gw];
     }

@@ -88,6 +88,194 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
+// old with lane LANE replaced by the wave-uniform value val (v_writelane_b32: one VALU operation)
+template <int LANE>
+__device__ __forceinline__ int write_lane(int val, int old) {
+  static_assert(LANE >= 0 && LANE < 64, "lane index");
+  asm("v_writelane_b32 %0, %1, %2" : "+v"(old) : "s"(val), "n"(LANE));
+  return old;
+}
+
+// Quantize-and-pack output stage that works straight from the accumulator registers (no transpose
+// through LDS).  In the matrix-core layout lane (li, g) holds column li of a 32x32 block and, in
+// register r, row 8*(r/4) + 4*g + r%4.  The channel (column) is therefore fixed per lane: its
+// thresholds live in registers, and a compare over the wave IS the ballot -- the 64-bit compare mask
+// of register r holds the 32 channel bits of two output rows (one per lane half).  For a 2-bit code
+// with sorted thresholds t0 <= t1 <= t2:  bit1 = v >= t1,  bit0 = v >= (bit1 ? t2 : t0): two
+// compares and one select per 64 outputs.  Codes of 3 or 4 bits binary-search a threshold table in
+// LDS, one compare per output bit (TABLE).  The masks are bit-reversed (channel c -> bit 31 - c%32)
+// and parked in the lane whose index is the output row; after a block is finished each lane stores
+// its row's words.  The four rows of a 2x2 pooling window (pool order) are the four registers
+// 4q..4q+3 of one lane, so pooling is register-local.
+//
+// Row-dependent terms come from LDS with 16-byte broadcast reads (four consecutive rows):
+//   lds[0 .. FA*32)                          activation row sums (convolution, symmetric weights)
+//   lds[FA*32 .. FA*32 + FA*2*FB*32)         shortcut words, index ((x*2 + plane)*FB + y)*32 + row
+//   lds[FA*32 + FA*64*FB ...)                threshold table [k][FB*32] (TABLE only), filled here
+template <bool F4, int FA, int FB, bool CONV, bool TABLE, class AccT>
+__device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA][FB],
+                                                const int (&ssum)[CONV ? FA : FB], uint32_t *lds, int rbase,
+                                                int cbase, int lane, const int (&T)[FB][3], const int (&fm)[FB],
+                                                bool shortcut) {
+  constexpr int NCOLS = FB * 32;
+  constexpr int NPARK = TABLE ? 2 : 1;
+  const int li = lane & 31, g = lane >> 5;
+  const int nb = p.out_bits;
+  const bool bn = p.epi == APNN_EPI_BN;
+  const int sh = p.sym ? 1 : 0;
+  const int wmax = p.sym ? p.wmax : 0;
+  const bool pooled = p.pool != APNN_POOL_NONE;
+  const int lowmask = (1 << nb) - 1;
+  const int bitpos = 31 - li;
+  const int w32 = p.rowsB >> 5;
+  const int *rowsum = reinterpret_cast<const int *>(lds);
+  const uint32_t *res = lds + FA * 32;
+  int *tl = reinterpret_cast<int *>(lds + FA * 32 + FA * 64 * FB);
+  if (TABLE && bn) {
+    const int nt = (1 << nb) - 1;
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      const int gcol = cbase + y * 32 + li;
+      if (gcol < p.rowsB)
+        for (int k = g; k < nt; k += 2) tl[k * NCOLS + y * 32 + li] = p.thr[(long long)gcol * nt + k];
+    }
+  }
+  int cneg[FB];  // GEMM entry points: the correction depends on the column only
+#pragma unroll
+  for (int y = 0; y < FB; ++y) cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
+
+  static_for<0, FA>([&](auto xc) {
+    constexpr int x = decltype(xc)::value;
+    uint32_t park[FB][NPARK];
+#pragma unroll
+    for (int y = 0; y < FB; ++y)
+#pragma unroll
+      for (int k = 0; k < NPARK; ++k) park[y][k] = 0;
+
+    static_for<0, 4>([&](auto qc) {
+      constexpr int q = decltype(qc)::value;
+      int negc[4] = {0, 0, 0, 0};
+      if (CONV) {
+        const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
+        negc[0] = -wmax * rs.x;
+        negc[1] = -wmax * rs.y;
+        negc[2] = -wmax * rs.z;
+        negc[3] = -wmax * rs.w;
+      }
+      static_for<0, FB>([&](auto yc) {
+        constexpr int y = decltype(yc)::value;
+        uint32_t rw[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        if (shortcut) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const uint4 w4 = *reinterpret_cast<const uint4 *>(res + ((x * 2 + b) * FB + y) * 32 + 8 * q + 4 * g);
+            rw[b][0] = w4.x;
+            rw[b][1] = w4.y;
+            rw[b][2] = w4.z;
+            rw[b][3] = w4.w;
+          }
+        }
+        int v[4];
+        static_for<0, 4>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          int t;
+          if constexpr (F4) {
+            t = __float2int_rn(acc[x][y][4 * q + j] * 4.0f);
+          } else {
+            t = acc[x][y][4 * q + j];
+          }
+          t = (t << sh) + (CONV ? negc[j] : cneg[y]);
+          if (shortcut) {
+            const int code = (int)(((rw[0][j] >> bitpos) & 1u) | (((rw[1][j] >> bitpos) & 1u) << 1));
+            t += code * p.resid_scale;
+          }
+          v[j] = t;
+        });
+        // one item: value (or code) -> one ballot per output bit, words parked at lanes rlo (lane
+        // half 0's row) and rhi (lane half 1's row)
+        auto emit = [&](int val, auto rlo_c, auto rhi_c) {
+          constexpr int rlo = decltype(rlo_c)::value, rhi = decltype(rhi_c)::value;
+          auto put = [&](auto slot_c, unsigned long long mask) {
+            constexpr int slot = decltype(slot_c)::value;
+            const int lo = (int)__brev((uint32_t)mask), hi = (int)__brev((uint32_t)(mask >> 32));
+            int reg = (int)park[y][slot >> 1];
+            reg = write_lane<rlo + 32 * (slot & 1)>(lo, reg);
+            reg = write_lane<rhi + 32 * (slot & 1)>(hi, reg);
+            park[y][slot >> 1] = (uint32_t)reg;
+          };
+          if (!bn) {
+            static_for<0, 2 * NPARK>([&](auto bc) {
+              constexpr int b = decltype(bc)::value;
+              if (b < nb) put(bc, __ballot((val >> b) & 1));
+            });
+          } else if constexpr (!TABLE) {
+            const bool hi1 = val >= T[y][1];
+            put(std::integral_constant<int, 1>{}, __ballot(hi1));
+            const int tsel = hi1 ? T[y][2] : T[y][0];
+            put(std::integral_constant<int, 0>{}, __ballot(val >= tsel));
+          } else {
+            int idx = (1 << (nb - 1)) - 1, h = 1 << (nb - 1);
+            static_for<0, 4>([&](auto lc) {
+              constexpr int lvl = decltype(lc)::value;
+              if (lvl < nb) {
+                h >>= 1;
+                const bool d = val >= tl[idx * NCOLS + y * 32 + li];
+                put(lc, __ballot(d));
+                idx += d ? h : -h;
+              }
+            });
+          }
+        };
+        auto flipped = [&](int t) { return (t ^ fm[y]) - fm[y]; };
+        if (!pooled) {
+          static_for<0, 4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            emit(bn ? flipped(v[j]) : (v[j] & lowmask), std::integral_constant<int, 8 * q + j>{},
+                 std::integral_constant<int, 8 * q + 4 + j>{});
+          });
+        } else {
+          int val;
+          if (p.pool == APNN_POOL_AVG2X2) {
+            const int a = (v[0] + v[1] + v[2] + v[3]) / 4;
+            val = bn ? flipped(a) : (a & lowmask);
+          } else if (bn) {
+            val = max(max(flipped(v[0]), flipped(v[1])), max(flipped(v[2]), flipped(v[3])));
+          } else {
+            val = max(max(v[0] & lowmask, v[1] & lowmask), max(v[2] & lowmask, v[3] & lowmask));
+          }
+          emit(val, std::integral_constant<int, 2 * q>{}, std::integral_constant<int, 2 * q + 1>{});
+        }
+      });
+    });
+
+    // lane L holds, in park[y][k], the word of block row L%32 for slot 2k + L/32
+    const int row = lane & 31;
+    const int rows_blk = pooled ? 8 : 32;
+    const int grow = (pooled ? (rbase >> 2) + x * 8 : rbase + x * 32) + row;
+    const int grow_end = pooled ? (p.rowsA >> 2) : p.rowsA;
+    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+    const int gw0 = cbase >> 5;
+#pragma unroll
+    for (int k = 0; k < NPARK; ++k) {
+      const int slot = 2 * k + (lane >> 5);
+      const int plane = (TABLE && bn) ? nb - 1 - slot : slot;
+      if (plane >= 0 && plane < nb && row < rows_blk && grow < grow_end && gw0 < w32) {
+        uint32_t *dst = out + plane * p.out_plane + (long long)grow * w32 + gw0;
+        if (FB == 4 && (w32 & 3) == 0) {
+          *reinterpret_cast<uint4 *>(dst) = make_uint4(park[0][k], park[FB > 1 ? 1 : 0][k], park[FB > 2 ? 2 : 0][k],
+                                                       park[FB > 3 ? 3 : 0][k]);
+        } else if (FB == 2 && (w32 & 1) == 0) {
+          *reinterpret_cast<uint2 *>(dst) = make_uint2(park[0][k], park[FB > 1 ? 1 : 0][k]);
+        } else {
+#pragma unroll
+          for (int y = 0; y < FB; ++y)
+            if (gw0 + y < w32) dst[y] = park[y][k];
+        }
+      }
+    }
+  });
+}
+
 // Output stage of one wave for a 32-row slab of its tile, staged in LDS as slab[32][NCOLS + 1]
 // (row-major, so the 64 lanes walk 64 consecutive output channels).  rowsum / colsum hold the
 // activation sums for the symmetric-weight correction (rows for convolution, columns for the GEMM
@@ -136,7 +324,7 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
     }
     return;
   }
-  if (p.out_bits <= 2 && p.resid == nullptr && p.save_acc == nullptr &&
+  if (KS > 1 && p.out_bits <= 2 && p.resid == nullptr && p.save_acc == nullptr &&
       (p.resid_planes == nullptr || res_lds != nullptr)) {
     pack_rows_burst<32, NCOLS, KS>(p, value, rbase, cbase, part, q0, q1, res_lds);
   } else {
@@ -297,18 +485,50 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
   for (int pl = 0; pl < PB; ++pl) rotB[pl] = (uint32_t)(4 * g - pl) & 31u;
 
-  // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop
+  // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop.
+  // Kernels whose waves tile the output (KS == 1) quantize straight from the accumulators when the
+  // epilogue allows it (`direct`); split-K kernels and the remaining epilogues go through the slab.
   constexpr int NCOLS_E = FB * 32;
   constexpr int RES_REGS = NCOLS_E / 32;  // two planes x 32 rows x NCOLS/32 words over 64 lanes
+  // (the 3- and 4-bit variant is built into the kernels whose activations have 3 or 4 planes)
+  constexpr int DIRECT_BITS = (CONV ? PA : PB) >= 3 ? 4 : 2;
+  const bool direct = KS == 1 && p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
+                      p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
   ChannelQuant q0{}, q1{};
+  int thrT[FB][3], flipm[FB];
   uint32_t res_regs[FA][RES_REGS];
   bool res_prefetched = false;
   if (p.epi != APNN_EPI_INT32) {
-    load_tile_quant<NCOLS_E>(p, b0 + wb * FB * 32, q0, q1);
-    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE) {
+    if (direct) {
 #pragma unroll
-      for (int x = 0; x < FA; ++x)
-        shortcut_prefetch<NCOLS_E, RES_REGS>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64, res_regs[x]);
+      for (int y = 0; y < FB; ++y) {
+        const int gcol = b0 + (wb * FB + y) * 32 + li;
+        thrT[y][0] = thrT[y][1] = thrT[y][2] = 0;
+        flipm[y] = 0;
+        if (p.epi == APNN_EPI_BN && gcol < p.rowsB) {
+          flipm[y] = (p.flip != nullptr && p.flip[gcol] != 0) ? -1 : 0;
+          if (p.out_bits <= 2) {
+            const int nt = (1 << p.out_bits) - 1;
+            const int32_t *t = p.thr + (long long)gcol * nt;
+            thrT[y][0] = t[0];
+            thrT[y][1] = nt > 1 ? t[1] : t[0];
+            thrT[y][2] = nt > 2 ? t[2] : t[0];
+          }
+        }
+      }
+    } else if (KS > 1) {
+      load_tile_quant<NCOLS_E>(p, b0 + wb * FB * 32, q0, q1);
+    }
+    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (direct || KS > 1)) {
+#pragma unroll
+      for (int x = 0; x < FA; ++x) {
+        if (KS == 1)
+          shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64,
+                                                     res_regs[x]);
+        else
+          shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64,
+                                                      res_regs[x]);
+      }
       res_prefetched = true;
     }
   }
@@ -464,7 +684,29 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   constexpr int NCOLS = FB * 32, LDT = NCOLS + 1;
   constexpr int RES_WORDS = 2 * 32 * (NCOLS / 32);
   constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS + RES_WORDS;
+  constexpr int DIRECT_WORDS = FA * 32 + FA * 64 * FB + 15 * NCOLS;
+  static_assert(DIRECT_WORDS <= SLAB_WORDS, "the register epilogue reuses the slab area");
   __syncthreads();  // every wave is done with the staging buffers
+  if constexpr (KS == 1) {
+    if (direct) {
+      uint32_t *area = smem + wave * SLAB_WORDS;
+      if (CONV && g == 0) {
+#pragma unroll
+        for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)ssum[CONV ? x : 0];
+      }
+      if (res_prefetched) {
+#pragma unroll
+        for (int x = 0; x < FA; ++x) shortcut_publish<RES_REGS>(area + FA * 32 + x * 64 * FB, lane, 64, res_regs[x]);
+      }
+      const int rb = a0 + wa * FA * 32, cb = b0 + wb * FB * 32;
+      if (DIRECT_BITS == 2 || p.out_bits <= 2) {
+        direct_epilogue<F4, FA, FB, CONV, false>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+      } else if constexpr (DIRECT_BITS > 2) {
+        direct_epilogue<F4, FA, FB, CONV, true>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+      }
+      return;
+    }
+  }
   int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
   int *rowsum = slab + 32 * LDT;
   int *colsum = rowsum + 32;

@@ -447,3 +447,65 @@ def test_pool_planes_wide_codes(G):
     G.A.check(G.A.lib().apnn_pool_planes(G.ptr(d_in), G.ptr(d_out), B, H, W, C, bits, 3, 2, 1, None), "pool_planes")
     pexp = O.pack_bits(pooled.reshape(prow, C).astype(np.uint32), prow, C, C, bits)
     assert np.array_equal(G.to_host(d_out, np.uint32).reshape(pexp.shape), pexp)
+
+
+# ---- quantizing epilogues without int32 side inputs (the register-resident output stage of the
+# ---- matrix-core kernels), every code width it serves ------------------------------------------------
+@pytest.mark.parametrize("mode", ["bn", "lowbits"])
+@pytest.mark.parametrize("pool", [0, 1, 2])
+@pytest.mark.parametrize("xb,ob", [(2, 1), (2, 2), (2, 3), (3, 3), (4, 4), (4, 1), (3, 2), (2, 4)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (1, None)])
+def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
+    rng = np.random.default_rng(4000 + 100 * xb + 10 * ob + pool + (tile or 0))
+    batch, H, Wd, C, cout, wb = 2, 6, 10, 64, 96, 1
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    sym = int(mode == "bn")
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=sym, **kw)
+    rows = batch * H * Wd if pool == 0 else batch * (H // 2) * (Wd // 2)
+    if mode == "bn":
+        span = int(np.abs(acc).max())
+        thr = np.sort(rng.integers(-span, span, size=(cout, 2 ** ob - 1)), axis=1).astype(np.int32)
+        thr[1] = thr[1, 0]                      # a channel whose thresholds coincide
+        flip = rng.integers(0, 2, size=cout).astype(np.uint8)
+        d_thr, d_flip = G.to_dev(thr), G.to_dev(flip)
+        epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, pool=pool, thr=d_thr, flip=d_flip)
+        if pool == 0:
+            q = O.bn_quantize(acc.reshape(-1, cout), None, thr, flip, ob)
+        elif pool == 1:
+            q = O.bn_quantize(O.avgpool2x2(acc).reshape(-1, cout), None, thr, flip, ob)
+        else:
+            q = O.maxpool2x2(O.bn_quantize(acc.reshape(-1, cout), None, thr, flip, ob).reshape(acc.shape)).reshape(-1, cout)
+    else:
+        epi = G.epilogue(mode=G.A.EPI_LOWBITS, out_bits=ob, pool=pool)
+        mask = (1 << ob) - 1
+        if pool == 0:
+            q = acc.reshape(-1, cout) & mask
+        elif pool == 1:
+            q = O.avgpool2x2(acc).reshape(-1, cout) & mask
+        else:
+            q = O.maxpool2x2(acc & mask).reshape(-1, cout)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=sym, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(ob, rows, cout // 32)
+    assert np.array_equal(got, O.lowbits_pack(q.astype(np.int32), rows, cout, ob))
+
+
+@pytest.mark.parametrize("sym", [0, 1])
+@pytest.mark.parametrize("wb,xb,ob", [(1, 2, 2), (1, 2, 1), (1, 3, 3), (1, 4, 4), (2, 2, 2), (1, 2, 4)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 6), (2, 5), (3, 2), (1, None)])
+def test_gemm_quantize_pack_all_widths(G, path, tile, wb, xb, ob, sym):
+    rng = np.random.default_rng(4100 + 100 * xb + 10 * ob + sym + (tile or 0))
+    M, N, K = 80, 192, 384
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, wb, xb, sym_w=sym)
+    lo, hi = int(acc.min()), int(acc.max())
+    thr = np.sort(rng.integers(lo, hi + 1, size=(N, 2 ** ob - 1)), axis=1).astype(np.int32)
+    flip = rng.integers(0, 2, size=N).astype(np.uint8)
+    thr[flip == 1] = -thr[flip == 1, ::-1]
+    d_thr, d_flip = G.to_dev(thr), G.to_dev(flip)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, flip=d_flip)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, epi=epi, path=path, tile=tile).view(np.uint32).reshape(ob, M, N // 32)
+    q = O.bn_quantize(acc, None, thr, flip, ob)
+    assert 0 < q.mean() < 2 ** ob - 1
+    assert np.array_equal(got, O.lowbits_pack(q, M, N, ob))
