@@ -3,6 +3,8 @@
 // of packed codes, code unpacking and the int8 classifier.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../include/apnn_tc.h"
 #include "dispatch.h"
 
@@ -308,6 +310,202 @@ __global__ __launch_bounds__(256) void conv_i8_c4_kernel(const int8_t *__restric
   }
 }
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for_n(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for_n<I + 1, N>(f);
+  }
+}
+
+// old with lane LANE replaced by the wave-uniform value val
+template <int LANE>
+__device__ __forceinline__ int write_lane_n(int val, int old) {
+  asm("v_writelane_b32 %0, %1, %2" : "+v"(old) : "s"(val), "n"(LANE));
+  return old;
+}
+
+// ---- int8 first convolution for images, filter rows taken straight from the image bytes ------------
+// In NHWC memory the S pixels x C channels under one filter row are S*C consecutive bytes, so K is laid
+// out per filter row as that byte run, padded with zero weights to whole 16-byte halves (HPR halves per
+// row); the halves of all R rows are numbered consecutively and k-step ks consumes halves 2ks (lane
+// half 0) and 2ks+1 (lane half 1).  The patch of a pixel group (32 consecutive output pixels of one
+// output row) is R image-row segments copied to LDS as aligned dwords -- no per-pixel repacking -- with
+// the zero point removed by an XOR (x - 128 == x ^ 0x80 as int8) and out-of-image dwords set to zero.
+// A lane's 16 operand bytes start at byte lead + pixel*stride*C + 16*half of its row segment: five
+// aligned dword reads and four v_alignbyte.  With NKS > 0 the wave keeps its 64 x (NKS*32) weight
+// block in registers for the whole (persistent) kernel; with NKS == 0 weights are read from LDS.
+// The epilogue is the compare-is-ballot scheme of the matrix-core kernels: per accumulator register
+// two compares and a select give both bit-plane masks of two output pixels.
+// Requires C <= 4, (W*C) % 4 == 0, X 4-byte aligned, bits <= 2, COUT % 32 == 0.
+template <int NKS>
+__global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                           const int32_t *__restrict__ thr,
+                                                           uint32_t *__restrict__ planes, int B, int H, int W, int C,
+                                                           int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
+                                                           int bits, uint32_t xor_mask, int HPR, int NDW, int PWD) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int NH = R * HPR;
+  const int nks = (NH + 1) / 2;
+  const int KB = nks * 32, KPL = KB + 16;
+  int8_t *wl = reinterpret_cast<int8_t *>(lds);  // [64][KPL]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 31, g = lane >> 5;
+  uint32_t *patch = reinterpret_cast<uint32_t *>(lds + 64 * KPL) + wave * (R * PWD);
+  const int co0 = blockIdx.y * 64;
+  const int SC = S * C;
+
+  for (int i = tid; i < 64 * KB; i += 256) {
+    const int co = co0 + i / KB, k = i % KB;
+    const int hh = k >> 4, r = hh / HPR, kk = (hh % HPR) * 16 + (k & 15);
+    wl[(i / KB) * KPL + k] = (co < COUT && r < R && kk < SC) ? Wt[((long long)co * R + r) * SC + kk] : (int8_t)0;
+  }
+  __syncthreads();
+
+  constexpr int NW = NKS > 0 ? NKS : 1;
+  v4i_t wreg[2][NW];
+  int koff[NW];  // byte offset of this lane's half of k-step ks inside the patch
+  if (NKS > 0) {
+#pragma unroll
+    for (int ks = 0; ks < NW; ++ks) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+        wreg[nb][ks] = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KPL + ks * 32 + g * 16);
+      const int hh = 2 * ks + g;
+      const int r = min(hh / HPR, R - 1);
+      koff[ks] = r * PWD * 4 + (hh % HPR) * 16;
+    }
+  }
+
+  const int nt = (1 << bits) - 1;
+  int t0[2], t1[2], t2[2];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int co = co0 + nb * 32 + li;
+    t0[nb] = t1[nb] = t2[nb] = 0x7fffffff;
+    if (co < COUT) {
+      t0[nb] = thr[co * nt];
+      t1[nb] = nt > 1 ? thr[co * nt + 1] : t0[nb];
+      t2[nb] = nt > 2 ? thr[co * nt + 2] : t0[nb];
+    }
+  }
+
+  const int gpr = (Wo + 31) / 32;
+  const long long ngroups = (long long)B * Ho * gpr;
+  const long long rows_total = (long long)B * Ho * Wo;
+  const int cw32 = COUT >> 5;
+  const int rowbytes = W * C;
+  const int npatch = R * NDW;
+  const int lane_bytes = li * stride * C;
+
+  for (long long group = (long long)blockIdx.x * 4 + wave; group < ngroups; group += (long long)gridDim.x * 4) {
+    const int gx = (int)(group % gpr);
+    const int oy = (int)((group / gpr) % Ho);
+    const int b = (int)(group / ((long long)gpr * Ho));
+    const int ox0 = gx * 32;
+    const int s0 = (ox0 * stride - pad) * C;
+    const int sbase = s0 & ~3;  // two's complement: rounds towards minus infinity
+    const int lead = s0 - sbase;
+    const uint8_t *img = X + (long long)b * H * rowbytes;
+    // ---- patch: R row segments of NDW dwords, eight per lane in flight ------------------------
+    for (int base = 0; base < npatch; base += 64 * 8) {
+      uint32_t raw[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * 64 + lane;
+        const int r = idx / NDW, d = idx - r * NDW;
+        const int iy = oy * stride - pad + r;
+        const int sb = sbase + 4 * d;
+        const bool ok = idx < npatch && iy >= 0 && iy < H && sb >= 0 && sb < rowbytes;
+        raw[j] = ok ? (*reinterpret_cast<const uint32_t *>(img + (long long)iy * rowbytes + sb) ^ xor_mask) : 0u;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * 64 + lane;
+        const int r = idx / NDW, d = idx - r * NDW;
+        if (idx < npatch) patch[r * PWD + d] = raw[j];
+      }
+    }
+
+    v16i_t acc[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][r] = 0;
+    const int a0 = lead + lane_bytes;
+    auto operand = [&](int byte_off) {
+      const int a = a0 + byte_off;
+      const uint32_t *wp = patch + (a >> 2);
+      const uint32_t sh = (uint32_t)a & 3u;
+      const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3], w4 = wp[4];
+      v4i_t af;
+      af[0] = (int)__builtin_amdgcn_alignbyte(w1, w0, sh);
+      af[1] = (int)__builtin_amdgcn_alignbyte(w2, w1, sh);
+      af[2] = (int)__builtin_amdgcn_alignbyte(w3, w2, sh);
+      af[3] = (int)__builtin_amdgcn_alignbyte(w4, w3, sh);
+      return af;
+    };
+    if (NKS > 0) {
+#pragma unroll
+      for (int ks = 0; ks < NW; ++ks) {
+        const v4i_t af = operand(koff[ks]);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, wreg[nb][ks], acc[nb], 0, 0, 0);
+      }
+    } else {
+      int r = 0, h = g;  // half index 2ks + g = r * HPR + h
+      while (h >= HPR) {
+        h -= HPR;
+        ++r;
+      }
+      for (int ks = 0; ks < nks; ++ks) {
+        const v4i_t af = operand(min(r, R - 1) * PWD * 4 + h * 16);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KPL + ks * 32 + g * 16);
+          acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[nb], 0, 0, 0);
+        }
+        h += 2;
+        while (h >= HPR) {
+          h -= HPR;
+          ++r;
+        }
+      }
+    }
+
+    // ---- thresholds -> bit-plane words, parked at lane = pixel (+32 for plane 1) -------------------
+    int park[2] = {0, 0};
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      static_for_n<0, 16>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        constexpr int rlo = 8 * (r >> 2) + (r & 3), rhi = rlo + 4;
+        const int v = acc[nb][r];
+        const bool hi1 = v >= t1[nb];
+        const unsigned long long m1 = __ballot(hi1);
+        const int tsel = hi1 ? t2[nb] : t0[nb];
+        const unsigned long long m0 = __ballot(v >= tsel);
+        int reg = park[nb];
+        reg = write_lane_n<rlo>((int)__brev((uint32_t)m0), reg);
+        reg = write_lane_n<rhi>((int)__brev((uint32_t)(m0 >> 32)), reg);
+        reg = write_lane_n<rlo + 32>((int)__brev((uint32_t)m1), reg);
+        reg = write_lane_n<rhi + 32>((int)__brev((uint32_t)(m1 >> 32)), reg);
+        park[nb] = reg;
+      });
+    }
+    const int ox = ox0 + li, plane = g;
+    if (ox < Wo && plane < bits) {
+      uint32_t *dst = planes + plane * rows_total * cw32 + (((long long)b * Ho + oy) * Wo + ox) * cw32 + (co0 >> 5);
+      if ((cw32 & 1) == 0) {
+        *reinterpret_cast<uint2 *>(dst) = make_uint2((uint32_t)park[0], (uint32_t)park[1]);
+      } else {
+        dst[0] = (uint32_t)park[0];
+        if (co0 + 32 < COUT) dst[1] = (uint32_t)park[1];
+      }
+    }
+  }
+}
+
 // ---- max-pool directly on bit-planes ----------------------------------------------------------------
 // in: [bits][B*H*W][cw] -> out: [bits][B*Ho*Wo][cw]; the maximum of two multi-bit codes is computed for
 // 32 channels at once with bitwise logic (compare from the top plane down).
@@ -468,6 +666,29 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
   const long long npix = (long long)B * Ho * Wo;
   const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
   dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
+  if (C <= 4 && planes != nullptr && codes == nullptr && acc_out == nullptr && bits <= 2 && (COUT % 32) == 0 &&
+      ((W * C) % 4) == 0 && (reinterpret_cast<uintptr_t>(X) & 3u) == 0 && (zero_point == 0 || zero_point == 128) &&
+      thr != nullptr) {
+    // image rows consumed as bytes (no repacking): see conv_i8_rows_kernel
+    const int HPR = (S * C + 15) / 16;
+    const int nks = (R * HPR + 1) / 2;
+    const int NDW = (3 + (31 * stride + S) * C + 3) / 4;
+    const int need = (3 + 31 * stride * C + 16 * (HPR - 1) + 20 + 3) / 4;
+    const int PWD = (need > NDW ? need : NDW) | 1;  // odd pitch
+    const size_t lds = (size_t)64 * (nks * 32 + 16) + 4 * (size_t)R * PWD * 4;
+    if (lds <= 64 * 1024) {
+      dim3 g2(grid.x > 1024 ? 1024 : grid.x, grid.y);
+      const uint32_t xm = zero_point == 128 ? 0x80808080u : 0u;
+      const uint8_t *Xu = reinterpret_cast<const uint8_t *>(X);
+      if (nks == 7)
+        hipLaunchKernelGGL(conv_i8_rows_kernel<7>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD);
+      else
+        hipLaunchKernelGGL(conv_i8_rows_kernel<0>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD);
+      return hipGetLastError();
+    }
+  }
   if (C <= 4) {
     // dword-per-pixel patch kernel, persistent over pixel groups: the filter block is staged once
     // per work-group

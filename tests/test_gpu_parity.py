@@ -398,13 +398,16 @@ def test_conv_packed_residual(G, path, tile):
     assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
 
 
-@pytest.mark.parametrize("R,stride,pad,H,cout,C", [(7, 2, 3, 40, 64, 3), (11, 4, 5, 67, 64, 3), (3, 1, 1, 9, 96, 4),
-                                                   (5, 2, 2, 33, 32, 1)])
-def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, cout, C):
+@pytest.mark.parametrize("R,stride,pad,H,Wd,cout,C", [
+    (7, 2, 3, 40, 43, 64, 3), (11, 4, 5, 67, 70, 64, 3), (3, 1, 1, 9, 12, 96, 4), (5, 2, 2, 33, 36, 32, 1),
+    # row length a multiple of 4 bytes: the kernel that consumes image rows as bytes
+    (7, 2, 3, 40, 44, 64, 3), (7, 2, 3, 75, 132, 128, 3), (11, 4, 5, 67, 72, 64, 3), (3, 2, 0, 20, 70, 32, 2),
+    (7, 4, 3, 39, 64, 64, 3)])
+def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, Wd, cout, C):
     """First layer with packed output, then max-pool on the bit-planes."""
-    rng = np.random.default_rng(990 + R)
+    rng = np.random.default_rng(990 + R + Wd)
     B, bits = 2, 2
-    Xu = rng.integers(0, 256, size=(B, H, H + 3, C)).astype(np.uint8)
+    Xu = rng.integers(0, 256, size=(B, H, Wd, C)).astype(np.uint8)
     Wt = rng.integers(-128, 128, size=(cout, R, R, C)).astype(np.int8)
     acc = O.conv_i8(Wt, (Xu.astype(np.int16) - 128).astype(np.int8), stride, pad)
     Ho, Wo = acc.shape[1], acc.shape[2]
@@ -414,14 +417,14 @@ def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, cout, C):
     dX, dW, dT = torch.from_numpy(Xu).cuda(), G.to_dev(Wt), G.to_dev(thr)
     rows = B * Ho * Wo
     d_planes = G.dev_empty_i32(bits * rows * cout // 32, fill=-7)
-    G.A.check(L.apnn_conv_i8_bn_pack(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_planes), B, H, H + 3, C, cout, R, R,
+    G.A.check(L.apnn_conv_i8_bn_pack(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_planes), B, H, Wd, C, cout, R, R,
                                      stride, pad, bits, 128, None), "conv_i8_bn_pack")
     expect = O.pack_bits(codes.reshape(rows, cout).astype(np.uint32), rows, cout, cout, bits)
     assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect)
     # the uint8-code / int32 outputs of the same kernel
     d_codes = torch.empty(rows * cout, dtype=torch.uint8, device="cuda")
     d_acc = G.dev_empty_i32(rows * cout, fill=-7)
-    G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, H + 3, C, cout, R, R,
+    G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, Wd, C, cout, R, R,
                                 stride, pad, bits, 128, None), "conv_i8_bn")
     assert np.array_equal(G.to_host(d_acc).reshape(acc.shape), acc)
     torch.cuda.synchronize()
@@ -433,6 +436,29 @@ def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, cout, C):
         G.A.check(L.apnn_pool_planes(G.ptr(d_planes), G.ptr(d_out), B, Ho, Wo, cout, bits, win, st, pd, None), "pool_planes")
         pexp = O.pack_bits(pooled.reshape(prow, cout).astype(np.uint32), prow, cout, cout, bits)
         assert np.array_equal(G.to_host(d_out, np.uint32).reshape(pexp.shape), pexp)
+
+
+@pytest.mark.parametrize("bits,zero_point", [(1, 128), (1, 0), (2, 0)])
+def test_conv_i8_bn_pack_signed_input_and_one_bit(G, bits, zero_point):
+    rng = np.random.default_rng(1200 + bits + zero_point)
+    B, H, Wd, C, cout, R, stride, pad = 3, 30, 52, 3, 64, 7, 2, 3
+    if zero_point:
+        Xraw = rng.integers(0, 256, size=(B, H, Wd, C)).astype(np.uint8)
+        Xs = (Xraw.astype(np.int16) - zero_point).astype(np.int8)
+    else:
+        Xs = rng.integers(-128, 128, size=(B, H, Wd, C)).astype(np.int8)
+        Xraw = Xs
+    Wt = rng.integers(-128, 128, size=(cout, R, R, C)).astype(np.int8)
+    acc = O.conv_i8(Wt, Xs, stride, pad)
+    rows = acc.shape[0] * acc.shape[1] * acc.shape[2]
+    thr = np.sort(rng.integers(-60000, 60000, size=(cout, 2 ** bits - 1)), axis=1).astype(np.int32)
+    codes = O.bn_quantize(acc.reshape(-1, cout), None, thr, None, bits)
+    dX, dW, dT = torch.from_numpy(Xraw).cuda(), G.to_dev(Wt), G.to_dev(thr)
+    d_planes = G.dev_empty_i32(bits * rows * cout // 32, fill=-7)
+    G.A.check(G.A.lib().apnn_conv_i8_bn_pack(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_planes), B, H, Wd, C, cout, R, R,
+                                             stride, pad, bits, zero_point, None), "conv_i8_bn_pack")
+    expect = O.pack_bits(codes.astype(np.uint32), rows, cout, cout, bits)
+    assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect)
 
 
 def test_pool_planes_wide_codes(G):
