@@ -355,10 +355,18 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   const int co0 = blockIdx.y * 64;
   const int SC = S * C;
 
-  for (int i = tid; i < 64 * KB; i += 256) {
-    const int co = co0 + i / KB, k = i % KB;
-    const int hh = k >> 4, r = hh / HPR, kk = (hh % HPR) * 16 + (k & 15);
-    wl[(i / KB) * KPL + k] = (co < COUT && r < R && kk < SC) ? Wt[((long long)co * R + r) * SC + kk] : (int8_t)0;
+  // filter block -> LDS, one 16-byte half per task (its byte loads are independent of each other)
+  for (int task = tid; task < 64 * nks * 2; task += 256) {
+    const int col = task / (nks * 2), hh = task - col * (nks * 2);
+    const int r = hh / HPR, hq = hh - r * HPR;
+    const int co = co0 + col;
+    const int nvalid = (co < COUT && r < R) ? min(max(SC - hq * 16, 0), 16) : 0;
+    const int8_t *src = Wt + ((long long)co * R + r) * SC + hq * 16;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (i < nvalid) w[i >> 2] |= (uint32_t)(uint8_t)src[i] << (8 * (i & 3));
+    *reinterpret_cast<uint4 *>(wl + col * KPL + hh * 16) = make_uint4(w[0], w[1], w[2], w[3]);
   }
   __syncthreads();
 
@@ -398,32 +406,75 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   const int npatch = R * NDW;
   const int lane_bytes = li * stride * C;
 
-  for (long long group = (long long)blockIdx.x * 4 + wave; group < ngroups; group += (long long)gridDim.x * 4) {
+  // Patch element idx = slot * 64 + lane is dword d of row segment r, the same for every group:
+  // (r, d) is decoded once.  The raw dwords of the next group are requested before the current
+  // group is computed (patches of up to 512 dwords; larger ones are staged in place).
+  constexpr int NSLOT = 8;
+  const bool prefetch = npatch <= 64 * NSLOT;
+  int rd[NSLOT];
+#pragma unroll
+  for (int j = 0; j < NSLOT; ++j) {
+    const int idx = j * 64 + lane;
+    const int r = idx / NDW;
+    rd[j] = idx < npatch ? ((r << 16) | (idx - r * NDW)) : -1;
+  }
+  uint32_t raw[NSLOT];
+  auto request = [&](long long grp, int base) {
+    const int gx = (int)(grp % gpr);
+    const int oy = (int)((grp / gpr) % Ho);
+    const int b = (int)(grp / ((long long)gpr * Ho));
+    const int sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
+    const uint8_t *img = X + (long long)b * H * rowbytes;
+#pragma unroll
+    for (int j = 0; j < NSLOT; ++j) {
+      int r, d;
+      bool ok;
+      if (base == 0) {
+        r = rd[j] >> 16;
+        d = rd[j] & 0xffff;
+        ok = rd[j] >= 0;
+      } else {
+        const int idx = base + j * 64 + lane;
+        r = idx / NDW;
+        d = idx - r * NDW;
+        ok = idx < npatch;
+      }
+      const int iy = oy * stride - pad + r;
+      const int sb = sbase + 4 * d;
+      ok = ok && iy >= 0 && iy < H && sb >= 0 && sb < rowbytes;
+      raw[j] = ok ? (*reinterpret_cast<const uint32_t *>(img + (long long)iy * rowbytes + sb) ^ xor_mask) : 0u;
+    }
+  };
+  auto publish = [&](int base) {
+#pragma unroll
+    for (int j = 0; j < NSLOT; ++j) {
+      if (base == 0) {
+        if (rd[j] >= 0) patch[(rd[j] >> 16) * PWD + (rd[j] & 0xffff)] = raw[j];
+      } else {
+        const int idx = base + j * 64 + lane;
+        const int r = idx / NDW;
+        if (idx < npatch) patch[r * PWD + (idx - r * NDW)] = raw[j];
+      }
+    }
+  };
+
+  const long long gstep = (long long)gridDim.x * 4;
+  long long group = (long long)blockIdx.x * 4 + wave;
+  if (prefetch && group < ngroups) request(group, 0);
+  for (; group < ngroups; group += gstep) {
     const int gx = (int)(group % gpr);
     const int oy = (int)((group / gpr) % Ho);
     const int b = (int)(group / ((long long)gpr * Ho));
     const int ox0 = gx * 32;
     const int s0 = (ox0 * stride - pad) * C;
-    const int sbase = s0 & ~3;  // two's complement: rounds towards minus infinity
-    const int lead = s0 - sbase;
-    const uint8_t *img = X + (long long)b * H * rowbytes;
-    // ---- patch: R row segments of NDW dwords, eight per lane in flight ------------------------
-    for (int base = 0; base < npatch; base += 64 * 8) {
-      uint32_t raw[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * 64 + lane;
-        const int r = idx / NDW, d = idx - r * NDW;
-        const int iy = oy * stride - pad + r;
-        const int sb = sbase + 4 * d;
-        const bool ok = idx < npatch && iy >= 0 && iy < H && sb >= 0 && sb < rowbytes;
-        raw[j] = ok ? (*reinterpret_cast<const uint32_t *>(img + (long long)iy * rowbytes + sb) ^ xor_mask) : 0u;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * 64 + lane;
-        const int r = idx / NDW, d = idx - r * NDW;
-        if (idx < npatch) patch[r * PWD + d] = raw[j];
+    const int lead = s0 - (s0 & ~3);
+    if (prefetch) {
+      publish(0);
+      if (group + gstep < ngroups) request(group + gstep, 0);
+    } else {
+      for (int base = 0; base < npatch; base += 64 * NSLOT) {
+        request(group, base);
+        publish(base);
       }
     }
 
@@ -677,7 +728,18 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
     const int PWD = (need > NDW ? need : NDW) | 1;  // odd pitch
     const size_t lds = (size_t)64 * (nks * 32 + 16) + 4 * (size_t)R * PWD * 4;
     if (lds <= 64 * 1024) {
-      dim3 g2(grid.x > 1024 ? 1024 : grid.x, grid.y);
+      // persistent grid: exactly as many work-groups as the device holds at once
+      auto kern = nks == 7 ? conv_i8_rows_kernel<7> : conv_i8_rows_kernel<0>;
+      int per_cu = 0, cus = 0, dev = 0;
+      hipError_t e = hipGetDevice(&dev);
+      if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e == hipSuccess)
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern), 256, lds);
+      if (e != hipSuccess) return e;
+      unsigned resident = (unsigned)(per_cu > 0 ? per_cu : 1) * (unsigned)(cus > 0 ? cus : 256);
+      const unsigned slices = grid.y > 0 ? grid.y : 1;
+      resident = resident / slices > 0 ? resident / slices : 1;
+      dim3 g2(grid.x > resident ? resident : grid.x, grid.y);
       const uint32_t xm = zero_point == 128 ? 0x80808080u : 0u;
       const uint8_t *Xu = reinterpret_cast<const uint8_t *>(X);
       if (nks == 7)
