@@ -637,25 +637,31 @@ __global__ __launch_bounds__(256) void pool_pack_kernel(const uint8_t *__restric
 // ---- packed codes -> int8 values (optionally summed over `group` consecutive rows) ---------------
 // planes: [bits][rows][cpad/32];  out[r][c] = (sum_{j<group} code[r*group + j][c]) >> shift, int8.
 // group = 1, shift = 0: plain unpacking.  group = H*W: global pooling of a feature map.
+// JP (a power of two <= 64) consecutive lanes share one output element and split its `group` rows;
+// their partial sums meet in a butterfly reduction.
 __global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restrict__ planes, int8_t *__restrict__ out,
                                                          long long rows_out, int group, int C, int cpad, int bits,
-                                                         int shift) {
+                                                         int shift, int JP) {
   const int cw = cpad >> 5;
   const long long rows_in = rows_out * group;
   const long long total = rows_out * C;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (long long)gridDim.x * blockDim.x) {
+  const int part = threadIdx.x & (JP - 1);
+  const long long nthreads = (long long)gridDim.x * blockDim.x;
+  // every lane of a JP-group runs the same number of iterations (the shuffles need all of them)
+  for (long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x; t / JP < total; t += nthreads) {
+    const long long i = t / JP;
     const long long r = i / C;
     const int c = (int)(i % C);
+    const int sh = 31 - (c & 31);
     int sum = 0;
-    for (int j = 0; j < group; ++j) {
+    for (int j = part; j < group; j += JP) {
       const long long rin = r * group + j;
       int code = 0;
-      for (int b = 0; b < bits; ++b)
-        code |= (int)((planes[b * rows_in * cw + rin * cw + (c >> 5)] >> (31 - (c & 31))) & 1u) << b;
+      for (int b = 0; b < bits; ++b) code |= (int)((planes[b * rows_in * cw + rin * cw + (c >> 5)] >> sh) & 1u) << b;
       sum += code;
     }
-    out[i] = (int8_t)min(127, sum >> shift);
+    for (int off = JP >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (part == 0) out[i] = (int8_t)min(127, sum >> shift);
   }
 }
 
@@ -815,10 +821,12 @@ hipError_t launch_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H
 
 hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad,
                              int bits, int shift, hipStream_t s) {
-  long long blocks = (rows_out * C + 255) / 256;
+  int JP = 1;
+  while (JP < 16 && JP * 2 <= group) JP *= 2;
+  long long blocks = (rows_out * C * JP + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   hipLaunchKernelGGL(unpack_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, s, planes, out, rows_out, group, C, cpad,
-                     bits, shift);
+                     bits, shift, JP);
   return hipGetLastError();
 }
 

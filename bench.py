@@ -233,8 +233,14 @@ def main():
                 iters = 200 if batch == 8 else 50
                 A.check(NL.apnn_net_bench(net, img.data_ptr(), lg.data_ptr(), 10, iters, 0, stream, ctypes.byref(ev),
                                           ctypes.byref(wall)), "apnn_net_bench")
-                nets["%s_w1a2_b%d" % (nm, batch)] = {"ms_per_forward": round(wall.value / iters, 4),
-                                                     "images_per_sec": round(batch * iters / wall.value * 1e3, 1)}
+                entry = {"ms_per_forward": round(wall.value / iters, 4),
+                         "images_per_sec": round(batch * iters / wall.value * 1e3, 1)}
+                # the same forward replayed as one HIP graph (no per-kernel launch from the host)
+                A.check(NL.apnn_net_bench(net, img.data_ptr(), lg.data_ptr(), 10, iters, 1, stream, ctypes.byref(ev),
+                                          ctypes.byref(wall)), "apnn_net_bench(graph)")
+                entry["graph_ms_per_forward"] = round(wall.value / iters, 4)
+                entry["graph_images_per_sec"] = round(batch * iters / wall.value * 1e3, 1)
+                nets["%s_w1a2_b%d" % (nm, batch)] = entry
                 NL.apnn_net_destroy(net)
         if nets:
             extra["networks"] = nets
