@@ -6,7 +6,7 @@ import subprocess
 __all__ = [
     "LIB_PATH", "lib", "build", "Epilogue", "GemmDesc", "ConvDesc", "ApnnError", "check",
     "EPI_INT32", "EPI_LOWBITS", "EPI_BN", "POOL_NONE", "POOL_AVG2X2", "POOL_MAX2X2",
-    "PATH_AUTO", "PATH_VALU", "PATH_MFMA", "PATH_MFMA_I8", "WEIGHT_UNSIGNED", "WEIGHT_SYMMETRIC",
+    "PATH_AUTO", "PATH_VALU", "PATH_MFMA", "PATH_MFMA_I8", "PATH_MFMA_PATCH", "WEIGHT_UNSIGNED", "WEIGHT_SYMMETRIC",
     "OK", "EINVAL", "ENULL", "EALIGN", "EUNSUPPORTED", "DECLARED_SYMBOLS",
 ]
 
@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(PKG_DIR, "lib", "libapnn_tc.so")
 
 EPI_INT32, EPI_LOWBITS, EPI_BN = 0, 1, 2
 POOL_NONE, POOL_AVG2X2, POOL_MAX2X2 = 0, 1, 2
-PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_MFMA_I8 = 0, 1, 2, 3
+PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_MFMA_I8, PATH_MFMA_PATCH = 0, 1, 2, 3, 4
 WEIGHT_UNSIGNED, WEIGHT_SYMMETRIC = 0, 1
 OK, EINVAL, ENULL, EALIGN, EUNSUPPORTED = 0, -1, -2, -3, -4
 

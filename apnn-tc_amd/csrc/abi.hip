@@ -115,6 +115,68 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   return nullptr;
 }
 
+typedef hipError_t (*patch_fn)(int, const KParams &, hipStream_t);
+patch_fn patch_conv_fn(int xb, int wb) {
+  if (xb == 2 && wb == 1) return apnn::patch_conv_2_1_x;
+  if (xb == 3 && wb == 1) return apnn::patch_conv_3_1_x;
+  if (xb == 4 && wb == 1) return apnn::patch_conv_4_1_x;
+  if (xb == 2 && wb == 2) return apnn::patch_conv_2_2_x;
+  return nullptr;
+}
+
+// Pixels of the padded frame that `rows` consecutive output rows of the implicit GEMM can span,
+// maximised over where the run starts.  With gr = b*Ho + oy counting output rows over the batch, the
+// padded-frame base of an output pixel is gr*stride*PWs + b*(PHs - Ho*stride)*PWs + ox*stride, and
+// along a run d(gr)*Wo + d(ox) = rows - 1; the filter window adds (R-1)*PWs + S.  In pool order a
+// row run is rows/4 consecutive 2x2 windows (window grid Ho/2 x Wo/2, step 2*stride) plus one
+// window's extent.
+int patch_pixels(const KParams &p, int R, int rows) {
+  const int st = p.pool_order ? 2 * p.stride : p.stride;
+  const int Wo = p.pool_order ? p.Wo / 2 : p.Wo, Ho = p.pool_order ? p.Ho / 2 : p.Ho;
+  const int n = p.pool_order ? rows / 4 : rows;
+  const int dgr = n > 1 ? (n - 2) / Wo + 1 : 0;            // output-row boundaries crossed, at most
+  const int db = dgr > 0 ? (dgr - 1) / Ho + 1 : 0;         // image boundaries crossed, at most
+  const int row_gap = st * (p.PWs - Wo) > 0 ? st * (p.PWs - Wo) : 0;
+  const int img_gap = (p.PHs - Ho * st) > 0 ? (p.PHs - Ho * st) * p.PWs : 0;
+  long long span = (long long)(n - 1) * st + (long long)dgr * row_gap + (long long)db * img_gap;
+  if (p.pool_order) span += p.stride * p.PWs + p.stride;
+  span += (long long)(R - 1) * p.PWs + p.S;
+  return span > 0x7fffffff ? 0x7fffffff : (int)span;
+}
+
+// Tile of the patch-resident convolution kernel, or -1 when it does not apply: the patch (at most
+// 1024 pixels) and the filter block of all taps must fit in LDS twice per compute unit, and -- when
+// the library chooses (`automatic`) -- there must be enough tiles to occupy the chip.
+int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;
+  const int taps = p.KW / p.C32;
+  auto fits = [&](int t) {
+    const int cap = patch_pixels(p, R, apnn::kPatchTileRows[t]);
+    if (cap > 1024) return false;
+    // digits: one per plane pair; the byte counts of patch_smem_bytes() for the widest case
+    const size_t bytes = ((size_t)2 * cap * 8 + (size_t)taps * apnn::kPatchTileCols[t] * 8 + cap) * 4;
+    return bytes <= 80 * 1024;
+  };
+  auto ntiles = [&](int t) {
+    return (long long)((p.rowsA + apnn::kPatchTileRows[t] - 1) / apnn::kPatchTileRows[t]) *
+           ((p.rowsB + apnn::kPatchTileCols[t] - 1) / apnn::kPatchTileCols[t]);
+  };
+  if (automatic && tile_pin != 0) return -1;  // a pinned tile names a tile of the implicit-GEMM families
+  if (tile_pin != 0) {
+    const int t = tile_pin - 1;
+    return (t < apnn::kPatchTileCount && fits(t)) ? t : -1;
+  }
+  const int narrow[3] = {1, 3, 4}, wide[3] = {0, 2, 4};  // 256x64,128x64,64x64 / 128x128,64x128,64x64
+  const int *cand = p.rowsB <= 64 ? narrow : wide;
+  for (int i = 0; i < 3; ++i)
+    if (fits(cand[i]) && ntiles(cand[i]) >= cus) return cand[i];
+  if (automatic) return -1;
+  for (int i = 2; i >= 0; --i)
+    if (fits(cand[i])) return cand[i];
+  return -1;
+}
+
 int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTED : (int)e; }
 
 // MFMA tile.  Large problems take the 256x128 (GEMM entry points) / 128x256 (convolution) shape: the
@@ -209,6 +271,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->D, d->M);
 
   int tile;
+  if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;
@@ -231,7 +294,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
-  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_I8))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_PATCH))
     return APNN_EINVAL;
   if (d->H + 2 * d->pad < d->R || d->Wd + 2 * d->pad < d->S) return APNN_EINVAL;
   const int Ho = (d->H + 2 * d->pad - d->R) / d->stride + 1;
@@ -268,6 +331,18 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
 
   int tile;
+  p.batch = d->batch;
+  p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
+  p.PWs = d->Wd + 2 * d->pad;
+  if (path == APNN_PATH_MFMA_PATCH || path == APNN_PATH_AUTO) {
+    patch_fn pf = patch_conv_fn(d->xb, d->wb);
+    const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
+    if (pt >= 0) {
+      p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
+      return from_hip(pf(pt, p, stream));
+    }
+    if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;
+  }
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
     if (fn == nullptr) return APNN_EUNSUPPORTED;

@@ -35,12 +35,23 @@ APNN_DECL_MFMA4(conv, 3, 1)
 APNN_DECL_MFMA4(conv, 4, 1)
 APNN_DECL_MFMA4(conv, 2, 2)
 #undef APNN_DECL_MFMA
+#define APNN_DECL_PATCH(pa, pb) hipError_t patch_conv_##pa##_##pb##_x(int tile, const KParams &p, hipStream_t s);
+APNN_DECL_PATCH(2, 1)
+APNN_DECL_PATCH(3, 1)
+APNN_DECL_PATCH(4, 1)
+APNN_DECL_PATCH(2, 2)
+#undef APNN_DECL_PATCH
 #undef APNN_DECL_MFMA4
 
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
 constexpr int kMfmaTileCount = 8;
 constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128};
 constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256};
+
+// tile shapes of the patch-resident convolution kernel, index = enum PatchTile in patch_conv_kernel.h
+constexpr int kPatchTileCount = 5;
+constexpr int kPatchTileRows[kPatchTileCount] = {128, 256, 64, 128, 64};
+constexpr int kPatchTileCols[kPatchTileCount] = {128, 64, 128, 64, 64};
 
 // aux_kernels.hip
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,

@@ -28,6 +28,10 @@ struct KParams {
   uint32_t magicC32, magicS; // ceil(2^32/d) for d >= 2 (unused when d == 1)
   int pool_order;            // 1: row index enumerates 2x2 output windows (4 consecutive rows each)
 
+  // patch-resident convolution kernel only: padded frame (stored frame + pad on every side) and
+  // the capacity of the LDS patch in pixels
+  int batch, PHs, PWs, patch_cap;
+
   int sym;                   // symmetric weights: result = 2*raw - wmax * (activation row sum)
   int wmax;                  // 2^wb - 1
 

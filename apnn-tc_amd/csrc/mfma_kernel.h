@@ -332,6 +332,150 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
   }
 }
 
+// Epilogue operands a wave requests before its K loop and consumes after it.
+template <int FA, int FB>
+struct EpiOperands {
+  bool direct;            // quantize straight from the accumulators (see direct_epilogue)
+  bool res_prefetched;    // shortcut words are in res_regs
+  ChannelQuant q0, q1;    // slab path (split-K kernels)
+  int thrT[FB][3], flipm[FB];
+  uint32_t res_regs[FA][FB];
+};
+
+// rbase / cbase: first output row / column of this wave's tile.  Kernels whose waves tile the output
+// (KS == 1) quantize straight from the accumulators when the epilogue allows it (`direct`; codes of up
+// to DIRECT_BITS bits); split-K kernels and the remaining epilogues go through the slab.
+template <int KS, int DIRECT_BITS, int FA, int FB>
+__device__ __forceinline__ void epi_prefetch(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
+  constexpr int NCOLS_E = FB * 32;
+  constexpr int RES_REGS = FB;  // two planes x 32 rows x NCOLS/32 words over 64 lanes
+  const int li = lane & 31;
+  eo.direct = KS == 1 && p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
+              p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
+  eo.q0 = ChannelQuant{};
+  eo.q1 = ChannelQuant{};
+  eo.res_prefetched = false;
+  if (p.epi != APNN_EPI_INT32) {
+    if (eo.direct) {
+#pragma unroll
+      for (int y = 0; y < FB; ++y) {
+        const int gcol = cbase + y * 32 + li;
+        eo.thrT[y][0] = eo.thrT[y][1] = eo.thrT[y][2] = 0;
+        eo.flipm[y] = 0;
+        if (p.epi == APNN_EPI_BN && gcol < p.rowsB) {
+          eo.flipm[y] = (p.flip != nullptr && p.flip[gcol] != 0) ? -1 : 0;
+          if (p.out_bits <= 2) {
+            const int nt = (1 << p.out_bits) - 1;
+            const int32_t *t = p.thr + (long long)gcol * nt;
+            eo.thrT[y][0] = t[0];
+            eo.thrT[y][1] = nt > 1 ? t[1] : t[0];
+            eo.thrT[y][2] = nt > 2 ? t[2] : t[0];
+          }
+        }
+      }
+    } else if (KS > 1) {
+      load_tile_quant<NCOLS_E>(p, cbase, eo.q0, eo.q1);
+    }
+    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (eo.direct || KS > 1)) {
+#pragma unroll
+      for (int x = 0; x < FA; ++x) {
+        if (KS == 1)
+          shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
+        else
+          shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
+      }
+      eo.res_prefetched = true;
+    }
+  }
+}
+
+// Output stage of a work-group of four waves (WA x WB of them tile the output, KS = 4 / (WA*WB) split
+// K).  acc: this wave's FA x FB accumulator blocks; ssum: activation sums of the lane's row li of each
+// row block (convolution) or column li of each column block (GEMM entry points), complete in every
+// lane.  smem: the work-group's LDS, free for reuse after the barrier at the top.
+template <bool F4, int KS, bool CONV, int DIRECT_BITS, int FA, int FB, class AccT>
+__device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB], const int (&ssum)[CONV ? FA : FB],
+                                           uint32_t *smem, int wave, int lane, int a0, int b0, int wa, int wb,
+                                           EpiOperands<FA, FB> &eo) {
+  const int li = lane & 31, g = lane >> 5;
+  constexpr int RES_REGS = FB;
+  const bool direct = eo.direct, res_prefetched = eo.res_prefetched;
+  ChannelQuant &q0 = eo.q0, &q1 = eo.q1;
+  auto &thrT = eo.thrT;
+  auto &flipm = eo.flipm;
+  auto &res_regs = eo.res_regs;
+  // ---- epilogue: one 32-row slab of the wave tile at a time through LDS ----------------------
+  // Accumulator indices are compile-time constants (static_for) so they stay in registers; the
+  // slab turns the matrix-core layout (register r of a block = row 8*(r/4) + 4*g + r%4, column li)
+  // into row-major order for coalesced stores and 64-channel ballots.
+  constexpr int NCOLS = FB * 32, LDT = NCOLS + 1;
+  constexpr int RES_WORDS = 2 * 32 * (NCOLS / 32);
+  constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS + RES_WORDS;
+  constexpr int DIRECT_WORDS = FA * 32 + FA * 64 * FB + 15 * NCOLS;
+  static_assert(DIRECT_WORDS <= SLAB_WORDS, "the register epilogue reuses the slab area");
+  __syncthreads();  // every wave is done with the staging buffers
+  if constexpr (KS == 1) {
+    if (direct) {
+      uint32_t *area = smem + wave * SLAB_WORDS;
+      if (CONV && g == 0) {
+#pragma unroll
+        for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)ssum[CONV ? x : 0];
+      }
+      if (res_prefetched) {
+#pragma unroll
+        for (int x = 0; x < FA; ++x) shortcut_publish<RES_REGS>(area + FA * 32 + x * 64 * FB, lane, 64, res_regs[x]);
+      }
+      const int rb = a0 + wa * FA * 32, cb = b0 + wb * FB * 32;
+      if (DIRECT_BITS == 2 || p.out_bits <= 2) {
+        direct_epilogue<F4, FA, FB, CONV, false>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+      } else if constexpr (DIRECT_BITS > 2) {
+        direct_epilogue<F4, FA, FB, CONV, true>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+      }
+      return;
+    }
+  }
+  int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
+  int *rowsum = slab + 32 * LDT;
+  int *colsum = rowsum + 32;
+  uint32_t *res_lds = reinterpret_cast<uint32_t *>(colsum + NCOLS);
+
+  if (!CONV && g == 0) {
+#pragma unroll
+    for (int y = 0; y < FB; ++y) colsum[y * 32 + li] = ssum[CONV ? 0 : y];
+  }
+  static_for<0, FA>([&](auto xc) {
+    constexpr int x = decltype(xc)::value;
+    if (CONV && g == 0) rowsum[li] = ssum[CONV ? x : 0];
+    if (res_prefetched) shortcut_publish<RES_REGS>(res_lds, lane, 64, res_regs[x]);
+    static_for<0, FB>([&](auto yc) {
+      constexpr int y = decltype(yc)::value;
+      static_for<0, 16>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        int v;
+        if constexpr (F4) {
+          v = __float2int_rn(acc[x][y][r] * 4.0f);
+        } else {
+          v = acc[x][y][r];
+        }
+        slab[(8 * (r >> 2) + 4 * g + (r & 3)) * LDT + y * 32 + li] = v;
+      });
+    });
+    if constexpr (KS > 1) {
+      // all KS partial slabs must be complete before any wave sums them
+      __syncthreads();
+      const int *base = reinterpret_cast<const int *>(smem);
+      wave_epilogue<NCOLS, CONV, KS>(p, base, base + 32 * LDT, base + 32 * LDT + 32, SLAB_WORDS, wave, a0, b0, lane,
+                                     q0, q1, res_prefetched ? res_lds : nullptr);
+    } else {
+      // LDS operations of one wave complete in order: the reads below see the writes above, and the
+      // next slab's writes come after these reads
+      wave_epilogue<NCOLS, CONV, 1>(p, slab, rowsum, colsum, 0, 0, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane,
+                                    q0, q1, res_prefetched ? res_lds : nullptr);
+    }
+  });
+}
+
+
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
 __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   // four waves per work-group: WA x WB of them tile the output, the remaining factor KS splits K
@@ -485,53 +629,9 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
 #pragma unroll
   for (int pl = 0; pl < PB; ++pl) rotB[pl] = (uint32_t)(4 * g - pl) & 31u;
 
-  // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop.
-  // Kernels whose waves tile the output (KS == 1) quantize straight from the accumulators when the
-  // epilogue allows it (`direct`); split-K kernels and the remaining epilogues go through the slab.
-  constexpr int NCOLS_E = FB * 32;
-  constexpr int RES_REGS = NCOLS_E / 32;  // two planes x 32 rows x NCOLS/32 words over 64 lanes
-  // (the 3- and 4-bit variant is built into the kernels whose activations have 3 or 4 planes)
-  constexpr int DIRECT_BITS = (CONV ? PA : PB) >= 3 ? 4 : 2;
-  const bool direct = KS == 1 && p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
-                      p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
-  ChannelQuant q0{}, q1{};
-  int thrT[FB][3], flipm[FB];
-  uint32_t res_regs[FA][RES_REGS];
-  bool res_prefetched = false;
-  if (p.epi != APNN_EPI_INT32) {
-    if (direct) {
-#pragma unroll
-      for (int y = 0; y < FB; ++y) {
-        const int gcol = b0 + (wb * FB + y) * 32 + li;
-        thrT[y][0] = thrT[y][1] = thrT[y][2] = 0;
-        flipm[y] = 0;
-        if (p.epi == APNN_EPI_BN && gcol < p.rowsB) {
-          flipm[y] = (p.flip != nullptr && p.flip[gcol] != 0) ? -1 : 0;
-          if (p.out_bits <= 2) {
-            const int nt = (1 << p.out_bits) - 1;
-            const int32_t *t = p.thr + (long long)gcol * nt;
-            thrT[y][0] = t[0];
-            thrT[y][1] = nt > 1 ? t[1] : t[0];
-            thrT[y][2] = nt > 2 ? t[2] : t[0];
-          }
-        }
-      }
-    } else if (KS > 1) {
-      load_tile_quant<NCOLS_E>(p, b0 + wb * FB * 32, q0, q1);
-    }
-    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (direct || KS > 1)) {
-#pragma unroll
-      for (int x = 0; x < FA; ++x) {
-        if (KS == 1)
-          shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64,
-                                                     res_regs[x]);
-        else
-          shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane, 64,
-                                                      res_regs[x]);
-      }
-      res_prefetched = true;
-    }
-  }
+  // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop
+  EpiOperands<FA, FB> eo;
+  epi_prefetch<KS, (CONV ? PA : PB) >= 3 ? 4 : 2>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
 
   // packed words of this lane's rows for one k-step
   uint32_t wA[FA][PA], wB[FB][PB];
@@ -677,75 +777,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
     ssum[x] = t;
   }
 
-  // ---- epilogue: one 32-row slab of the wave tile at a time through LDS ----------------------
-  // Accumulator indices are compile-time constants (static_for) so they stay in registers; the
-  // slab turns the matrix-core layout (register r of a block = row 8*(r/4) + 4*g + r%4, column li)
-  // into row-major order for coalesced stores and 64-channel ballots.
-  constexpr int NCOLS = FB * 32, LDT = NCOLS + 1;
-  constexpr int RES_WORDS = 2 * 32 * (NCOLS / 32);
-  constexpr int SLAB_WORDS = 32 * LDT + 32 + NCOLS + RES_WORDS;
-  constexpr int DIRECT_WORDS = FA * 32 + FA * 64 * FB + 15 * NCOLS;
-  static_assert(DIRECT_WORDS <= SLAB_WORDS, "the register epilogue reuses the slab area");
-  __syncthreads();  // every wave is done with the staging buffers
-  if constexpr (KS == 1) {
-    if (direct) {
-      uint32_t *area = smem + wave * SLAB_WORDS;
-      if (CONV && g == 0) {
-#pragma unroll
-        for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)ssum[CONV ? x : 0];
-      }
-      if (res_prefetched) {
-#pragma unroll
-        for (int x = 0; x < FA; ++x) shortcut_publish<RES_REGS>(area + FA * 32 + x * 64 * FB, lane, 64, res_regs[x]);
-      }
-      const int rb = a0 + wa * FA * 32, cb = b0 + wb * FB * 32;
-      if (DIRECT_BITS == 2 || p.out_bits <= 2) {
-        direct_epilogue<F4, FA, FB, CONV, false>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
-      } else if constexpr (DIRECT_BITS > 2) {
-        direct_epilogue<F4, FA, FB, CONV, true>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
-      }
-      return;
-    }
-  }
-  int *slab = reinterpret_cast<int *>(smem) + wave * SLAB_WORDS;
-  int *rowsum = slab + 32 * LDT;
-  int *colsum = rowsum + 32;
-  uint32_t *res_lds = reinterpret_cast<uint32_t *>(colsum + NCOLS);
-
-  if (!CONV && g == 0) {
-#pragma unroll
-    for (int y = 0; y < FB; ++y) colsum[y * 32 + li] = ssum[CONV ? 0 : y];
-  }
-  static_for<0, FA>([&](auto xc) {
-    constexpr int x = decltype(xc)::value;
-    if (CONV && g == 0) rowsum[li] = ssum[CONV ? x : 0];
-    if (res_prefetched) shortcut_publish<RES_REGS>(res_lds, lane, 64, res_regs[x]);
-    static_for<0, FB>([&](auto yc) {
-      constexpr int y = decltype(yc)::value;
-      static_for<0, 16>([&](auto rc) {
-        constexpr int r = decltype(rc)::value;
-        int v;
-        if constexpr (F4) {
-          v = __float2int_rn(acc[x][y][r] * 4.0f);
-        } else {
-          v = acc[x][y][r];
-        }
-        slab[(8 * (r >> 2) + 4 * g + (r & 3)) * LDT + y * 32 + li] = v;
-      });
-    });
-    if constexpr (KS > 1) {
-      // all KS partial slabs must be complete before any wave sums them
-      __syncthreads();
-      const int *base = reinterpret_cast<const int *>(smem);
-      wave_epilogue<NCOLS, CONV, KS>(p, base, base + 32 * LDT, base + 32 * LDT + 32, SLAB_WORDS, wave, a0, b0, lane,
-                                     q0, q1, res_prefetched ? res_lds : nullptr);
-    } else {
-      // LDS operations of one wave complete in order: the reads below see the writes above, and the
-      // next slab's writes come after these reads
-      wave_epilogue<NCOLS, CONV, 1>(p, slab, rowsum, colsum, 0, 0, a0 + (wa * FA + x) * 32, b0 + wb * FB * 32, lane,
-                                    q0, q1, res_prefetched ? res_lds : nullptr);
-    }
-  });
+  epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
 }
 
 constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB) {

@@ -1,0 +1,281 @@
+// Patch-resident convolution on the matrix cores (FP4 operands, see mfma_kernel.h for the encoding).
+//
+// The implicit-GEMM kernel in mfma_kernel.h gathers, for every filter tap, the packed activation
+// words of every output pixel of its tile and expands them to matrix-core operands in registers --
+// R*S times per input pixel and once more per column tile.  Here the input pixels a tile needs are
+// expanded ONCE into LDS and every tap reads them in place:
+//
+//   * In the zero-padded frame (stored frame plus `pad` pixels on every side, PHs x PWs per image) the
+//     input pixel of output pixel (b, oy, ox) and tap (r, s) has the linear index
+//         q = (b*PHs + oy*stride)*PWs + ox*stride  +  r*PWs + s,
+//     i.e. a per-pixel base plus a per-tap constant.  A tile of consecutive output pixels therefore
+//     needs one contiguous range [q_lo, q_hi] of padded-frame pixels: the patch.
+//   * Per chunk of 64 channels the work-group stages the patch (bit-plane words -> FP4 digit
+//     operands, 16 bytes per pixel, 32-channel word and digit; padding pixels are zeros) and the
+//     filter block of its output channels for all taps (same encoding), then runs
+//     taps k-steps of pure LDS reads + MFMA:  A operand = patch[base(row) + tap offset], B operand =
+//     filter[tap][column].
+//   * Per-pixel activation sums (for the symmetric-weight correction) are taken once per patch pixel
+//     while staging; a row's window sum is the sum over taps of those.
+//
+// Output stage, tile-to-row mapping, epilogue operands and all quantizing modes are the ones of the
+// implicit-GEMM kernel (epi_prefetch / epi_finish).
+#pragma once
+#include "mfma_kernel.h"
+
+namespace apnn {
+
+constexpr int PATCH_NPT = 4;  // patch pixels per thread (patch capacity = 4 * 256 pixels)
+
+template <int PA, int PB, int FA, int FB, int WA, int WB, int OCC>
+__global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams p) {
+  static_assert(WA * WB == 4, "four waves tile the output");
+  constexpr int DA = (PA + 1) / 2, DB = (PB + 1) / 2;
+  constexpr int NT = 256;
+  constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
+  constexpr int DIRECT_BITS = PA >= 3 ? 4 : 2;
+
+  extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 31, g = lane >> 5;
+  const int wa = wave / WB, wb = wave % WB;
+  const int tilesB = (p.rowsB + TB - 1) / TB;
+  const int a0 = (blockIdx.x / tilesB) * TA;
+  const int b0 = (blockIdx.x % tilesB) * TB;
+  const int taps = p.KW / p.C32;
+  const int cap = p.patch_cap;
+
+  uint32_t *patchA = smem;                                 // [DA][cap][2 words][4 dwords]
+  uint32_t *filtB = patchA + DA * cap * 8;                 // [DB][taps][TB][2 words][4 dwords]
+  int *pixsum = reinterpret_cast<int *>(filtB + DB * taps * TB * 8);  // [cap]
+
+  // padded-frame base index of an output row of the tile
+  auto row_base = [&](int grow) {
+    int oy, ox, b;
+    if (p.pool_order) {
+      const int win = grow >> 2, sub = grow & 3;
+      const int hw = p.Wo >> 1, hh = p.Ho >> 1;
+      const int px = win % hw, t = win / hw;
+      const int py = t % hh;
+      b = t / hh;
+      oy = 2 * py + (sub >> 1);
+      ox = 2 * px + (sub & 1);
+    } else {
+      ox = grow % p.Wo;
+      const int t = grow / p.Wo;
+      oy = t % p.Ho;
+      b = t / p.Ho;
+    }
+    return (b * p.PHs + oy * p.stride) * p.PWs + ox * p.stride;
+  };
+  const int last_row = min(a0 + TA, p.rowsA) - 1;
+  const int R = taps / p.S;
+  const int q_lo = row_base(a0);
+  const int q_hi = row_base(last_row) + (R - 1) * p.PWs + (p.S - 1);
+  const int npp = q_hi - q_lo + 1;
+  if (npp > cap) return;  // the host sizes the patch for the worst tile; never taken
+
+  // this lane's rows: patch-relative pixel index of row li of each of its FA row blocks
+  int prow[FA];
+#pragma unroll
+  for (int x = 0; x < FA; ++x) prow[x] = row_base(min(a0 + (wa * FA + x) * 32 + li, last_row)) - q_lo;
+
+  // patch pixels this thread stages: global word offset of the pixel (channel word 0), or -1 for
+  // padding / beyond the range
+  long long poff[PATCH_NPT];
+  const int pad_v = (p.PHs - p.Hs) >> 1;
+  const int frame = p.PHs * p.PWs;
+#pragma unroll
+  for (int j = 0; j < PATCH_NPT; ++j) {
+    const int q = tid + j * NT;
+    poff[j] = -1;
+    if (q < npp) {
+      const int qq = q_lo + q;
+      const int img = qq / frame, rem = qq - img * frame;
+      const int yp = rem / p.PWs, xp = rem - yp * p.PWs;
+      const int iy = yp - pad_v, ix = xp - pad_v;
+      if (img < p.batch && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws)
+        poff[j] = (((long long)img * p.Hs + iy) * p.Ws + ix) * p.C32;
+    }
+  }
+
+  v16f acc[FA][FB];
+#pragma unroll
+  for (int x = 0; x < FA; ++x)
+#pragma unroll
+    for (int y = 0; y < FB; ++y)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[x][y][r] = 0;
+  int ssum[FA];
+#pragma unroll
+  for (int x = 0; x < FA; ++x) ssum[x] = 0;
+
+  EpiOperands<FA, FB> eo;
+  epi_prefetch<1, DIRECT_BITS>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
+
+  const bool pair_ok = (p.C32 & 1) == 0;  // 64-bit loads of a channel-word pair
+  const int nchunks = (p.C32 + 1) >> 1;
+  for (int cc = 0; cc < nchunks; ++cc) {
+    const int cw = cc * 2;
+    if (cc > 0) __syncthreads();  // every wave has finished reading the previous chunk
+    // ---- patch chunk: packed words -> FP4 digit operands --------------------------------------
+#pragma unroll
+    for (int j = 0; j < PATCH_NPT; ++j) {
+      const int q = tid + j * NT;
+      if (q < npp) {
+        uint32_t w0[PA], w1[PA];
+        const bool in = poff[j] >= 0;
+#pragma unroll
+        for (int pl = 0; pl < PA; ++pl) {
+          w0[pl] = w1[pl] = 0;
+          if (in) {
+            const uint32_t *src = p.A + pl * p.planeA + poff[j] + cw;
+            if (pair_ok) {
+              const uint2 v = *reinterpret_cast<const uint2 *>(src);
+              w0[pl] = v.x;
+              w1[pl] = v.y;
+            } else {
+              w0[pl] = src[0];
+              if (cw + 1 < p.C32) w1[pl] = src[1];
+            }
+          }
+        }
+        int ps = 0;
+#pragma unroll
+        for (int pl = 0; pl < PA; ++pl) ps += (__popc(w0[pl]) + __popc(w1[pl])) << pl;
+        pixsum[q] = ps;
+        static_for<0, DA>([&](auto dc) {
+          constexpr int d = decltype(dc)::value;
+          const v8i e0 = expand_fp4<PA, d>(w0), e1 = expand_fp4<PA, d>(w1);
+          uint4 *dst = reinterpret_cast<uint4 *>(patchA + ((d * cap + q) * 2) * 4);
+          dst[0] = make_uint4((uint32_t)e0[0], (uint32_t)e0[1], (uint32_t)e0[2], (uint32_t)e0[3]);
+          dst[1] = make_uint4((uint32_t)e1[0], (uint32_t)e1[1], (uint32_t)e1[2], (uint32_t)e1[3]);
+        });
+      }
+    }
+    // ---- filter chunk ----------------------------------------------------------------------
+    for (int t = tid; t < taps * TB; t += NT) {
+      const int tap = t / TB, col = t % TB;
+      const int gcol = b0 + col;
+      uint32_t w0[PB], w1[PB];
+#pragma unroll
+      for (int pl = 0; pl < PB; ++pl) {
+        w0[pl] = w1[pl] = 0;
+        if (gcol < p.rowsB) {
+          const uint32_t *src = p.B + pl * p.planeB + ((long long)gcol * taps + tap) * p.C32 + cw;
+          if (pair_ok) {
+            const uint2 v = *reinterpret_cast<const uint2 *>(src);
+            w0[pl] = v.x;
+            w1[pl] = v.y;
+          } else {
+            w0[pl] = src[0];
+            if (cw + 1 < p.C32) w1[pl] = src[1];
+          }
+        }
+      }
+      static_for<0, DB>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        const v8i e0 = expand_fp4<PB, d>(w0), e1 = expand_fp4<PB, d>(w1);
+        uint4 *dst = reinterpret_cast<uint4 *>(filtB + (((d * taps + tap) * TB + col) * 2) * 4);
+        dst[0] = make_uint4((uint32_t)e0[0], (uint32_t)e0[1], (uint32_t)e0[2], (uint32_t)e0[3]);
+        dst[1] = make_uint4((uint32_t)e1[0], (uint32_t)e1[1], (uint32_t)e1[2], (uint32_t)e1[3]);
+      });
+    }
+    __syncthreads();
+
+    // ---- taps k-steps: operands straight from LDS --------------------------------------------
+    int r = 0, sx = 0;
+    for (int tap = 0; tap < taps; ++tap) {
+      const int toff = r * p.PWs + sx;
+      v8i af[FA][DA], bf[FB][DB];
+#pragma unroll
+      for (int x = 0; x < FA; ++x) {
+        const int pix = prow[x] + toff;
+        ssum[x] += pixsum[pix];
+#pragma unroll
+        for (int d = 0; d < DA; ++d) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(patchA + ((d * cap + pix) * 2 + g) * 4);
+          af[x][d] = v8i{(int)v.x, (int)v.y, (int)v.z, (int)v.w, 0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int y = 0; y < FB; ++y) {
+#pragma unroll
+        for (int d = 0; d < DB; ++d) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(
+              filtB + (((d * taps + tap) * TB + (wb * FB + y) * 32 + li) * 2 + g) * 4);
+          bf[y][d] = v8i{(int)v.x, (int)v.y, (int)v.z, (int)v.w, 0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int x = 0; x < FA; ++x)
+#pragma unroll
+        for (int y = 0; y < FB; ++y) {
+          static_for<0, DA>([&](auto dac) {
+            static_for<0, DB>([&](auto dbc) {
+              constexpr int da = decltype(dac)::value, db = decltype(dbc)::value;
+              if constexpr (da + db == 0) {
+                acc[x][y] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[x][da], bf[y][db], acc[x][y], 4, 4, 0,
+                                                                            0, 0, 0);
+              } else {
+                acc[x][y] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    af[x][da], bf[y][db], acc[x][y], 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F + 0x02020202 * (da + db));
+              }
+            });
+          });
+        }
+      if (++sx == p.S) {
+        sx = 0;
+        ++r;
+      }
+    }
+  }
+  epi_finish<true, 1, true, DIRECT_BITS>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
+}
+
+// LDS bytes of a launch: patch + filter block + pixel sums, at least the slab area of the output stage
+constexpr size_t patch_smem_bytes(int PA, int PB, int FB, int TB, int taps, int cap) {
+  const size_t da = (PA + 1) / 2, db = (PB + 1) / 2;
+  const size_t stage = (da * cap * 8 + db * (size_t)taps * TB * 8 + cap) * sizeof(uint32_t);
+  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
+  return stage > slab ? stage : slab;
+}
+
+enum PatchTile { PT_128x128 = 0, PT_256x64 = 1, PT_64x128 = 2, PT_128x64 = 3, PT_64x64 = 4, PT_COUNT = 5 };
+constexpr int kPatchTileA[PT_COUNT] = {128, 256, 64, 128, 64};
+constexpr int kPatchTileB[PT_COUNT] = {128, 64, 128, 64, 64};
+
+template <int PA, int PB, int FA, int FB, int WA, int WB>
+inline hipError_t launch_patch(const KParams &p, hipStream_t stream) {
+  constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
+  const int taps = p.KW / p.C32;
+  const size_t smem_bytes = patch_smem_bytes(PA, PB, FB, TB, taps, p.patch_cap);
+  if (smem_bytes > 160 * 1024 || p.patch_cap > PATCH_NPT * 256) return hipErrorNotSupported;
+  auto kern = apnn_patch_conv_kernel<PA, PB, FA, FB, WA, WB, 2>;
+  if (smem_bytes > 64 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      raised = true;
+    }
+  }
+  const long long tiles = (long long)((p.rowsA + TA - 1) / TA) * ((p.rowsB + TB - 1) / TB);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), smem_bytes, stream, p);
+  return hipGetLastError();
+}
+
+template <int PA, int PB>
+inline hipError_t launch_patch_tile(int tile, const KParams &p, hipStream_t stream) {
+  switch (tile) {
+    case PT_128x128: return launch_patch<PA, PB, 2, 2, 2, 2>(p, stream);
+    case PT_256x64: return launch_patch<PA, PB, 2, 2, 4, 1>(p, stream);
+    case PT_64x128: return launch_patch<PA, PB, 1, 2, 2, 2>(p, stream);
+    case PT_128x64: return launch_patch<PA, PB, 1, 2, 4, 1>(p, stream);
+    case PT_64x64: return launch_patch<PA, PB, 1, 1, 2, 2>(p, stream);
+    default: return hipErrorNotSupported;
+  }
+}
+
+}  // namespace apnn

@@ -90,7 +90,10 @@ enum { APNN_POOL_NONE = 0,
 enum { APNN_PATH_AUTO = 0,
        APNN_PATH_VALU = 1,     /* v_and + v_bcnt popcount on packed words                           */
        APNN_PATH_MFMA = 2,     /* planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4      */
-       APNN_PATH_MFMA_I8 = 3 };/* planes expanded to int8 operands of v_mfma_i32_32x32x32_i8         */
+       APNN_PATH_MFMA_I8 = 3,  /* planes expanded to int8 operands of v_mfma_i32_32x32x32_i8         */
+       APNN_PATH_MFMA_PATCH = 4 };/* convolution only: FP4 matrix-core path with the tile's input patch
+                                  expanded once into LDS and read in place by every filter tap;
+                                  APNN_EUNSUPPORTED when the patch or filter block does not fit   */
 /* `path` fields: low byte = APNN_PATH_*; bits 8..15 = 0 (library picks the tile shape) or
  * 1 + tile index to pin it (tuning / test coverage of every tile shape; APNN_EINVAL if the
  * chosen kernel family has no such tile or the epilogue cannot use it). */

@@ -51,11 +51,11 @@ def test_gemm_named_entry_golden(G, wb, xb):
 
 
 PATHS = [1, 2, 3]   # APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8 (GEMM entry points only)
-CONV_PATHS = [1, 2]
+CONV_PATHS = [1, 2, 4]   # 4 = APNN_PATH_MFMA_PATCH (input patch resident in LDS)
 # (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
 # int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128
 GEMM_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)]
-CONV_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)]
+CONV_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)] + [(4, t) for t in range(5)]
 GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
 CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
 
@@ -480,7 +480,7 @@ def test_pool_planes_wide_codes(G):
 @pytest.mark.parametrize("mode", ["bn", "lowbits"])
 @pytest.mark.parametrize("pool", [0, 1, 2])
 @pytest.mark.parametrize("xb,ob", [(2, 1), (2, 2), (2, 3), (3, 3), (4, 4), (4, 1), (3, 2), (2, 4)])
-@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (1, None)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (1, None), (4, 0), (4, 1), (4, 4)])
 def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
     rng = np.random.default_rng(4000 + 100 * xb + 10 * ob + pool + (tile or 0))
     batch, H, Wd, C, cout, wb = 2, 6, 10, 64, 96, 1
