@@ -145,8 +145,10 @@ int patch_pixels(const KParams &p, int R, int rows) {
 }
 
 // Tile of the patch-resident convolution kernel, or -1 when it does not apply: the patch (at most
-// 1024 pixels) and the filter block of all taps must fit in LDS twice per compute unit, and -- when
-// the library chooses (`automatic`) -- there must be enough tiles to occupy the chip.
+// 1024 pixels) and the filter block of all taps must fit in LDS twice per compute unit.  When the
+// library chooses (`automatic`) the kernel is taken only where it measures faster than the
+// implicit-GEMM kernel: at most 64 output channels over at most 64 input channels (one channel
+// chunk, e.g. the first stage of ResNet18) with enough 128x64 tiles to occupy the chip.
 int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -162,16 +164,19 @@ int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
     return (long long)((p.rowsA + apnn::kPatchTileRows[t] - 1) / apnn::kPatchTileRows[t]) *
            ((p.rowsB + apnn::kPatchTileCols[t] - 1) / apnn::kPatchTileCols[t]);
   };
-  if (automatic && tile_pin != 0) return -1;  // a pinned tile names a tile of the implicit-GEMM families
+  if (automatic) {
+    if (tile_pin != 0) return -1;  // a pinned tile names a tile of the implicit-GEMM families
+    const int t = 3;               // 128 x 64
+    return (p.rowsB <= 64 && p.C32 <= 2 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus) ? t : -1;
+  }
   if (tile_pin != 0) {
     const int t = tile_pin - 1;
     return (t < apnn::kPatchTileCount && fits(t)) ? t : -1;
   }
-  const int narrow[3] = {1, 3, 4}, wide[3] = {0, 2, 4};  // 256x64,128x64,64x64 / 128x128,64x128,64x64
+  const int narrow[3] = {3, 1, 4}, wide[3] = {2, 0, 4};  // 128x64, 256x64, 64x64 / 64x128, 128x128, 64x64
   const int *cand = p.rowsB <= 64 ? narrow : wide;
   for (int i = 0; i < 3; ++i)
     if (fits(cand[i]) && ntiles(cand[i]) >= cus) return cand[i];
-  if (automatic) return -1;
   for (int i = 2; i >= 0; --i)
     if (fits(cand[i])) return cand[i];
   return -1;
@@ -339,6 +344,10 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
     if (pt >= 0) {
       p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
+      p.magicGW = magic_of(p.pool_order ? Wo / 2 : Wo);
+      p.magicGH = magic_of(p.pool_order ? Ho / 2 : Ho);
+      p.magicPW = magic_of(p.PWs);
+      p.magicPH = magic_of(p.PHs);
       return from_hip(pf(pt, p, stream));
     }
     if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;

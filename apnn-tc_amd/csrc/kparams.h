@@ -31,6 +31,9 @@ struct KParams {
   // patch-resident convolution kernel only: padded frame (stored frame + pad on every side) and
   // the capacity of the LDS patch in pixels
   int batch, PHs, PWs, patch_cap;
+  // ceil(2^32/d) for the row grid (Wo, Ho; in pool order Wo/2, Ho/2) and the padded frame (PWs, PHs):
+  // exact quotients for dividends below d + 1024
+  uint32_t magicGW, magicGH, magicPW, magicPH;
 
   int sym;                   // symmetric weights: result = 2*raw - wmax * (activation row sum)
   int wmax;                  // 2^wb - 1

@@ -49,50 +49,57 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
   uint32_t *filtB = patchA + DA * cap * 8;                 // [DB][taps][TB][2 words][4 dwords]
   int *pixsum = reinterpret_cast<int *>(filtB + DB * taps * TB * 8);  // [cap]
 
-  // padded-frame base index of an output row of the tile
-  auto row_base = [&](int grow) {
-    int oy, ox, b;
-    if (p.pool_order) {
-      const int win = grow >> 2, sub = grow & 3;
-      const int hw = p.Wo >> 1, hh = p.Ho >> 1;
-      const int px = win % hw, t = win / hw;
-      const int py = t % hh;
-      b = t / hh;
-      oy = 2 * py + (sub >> 1);
-      ox = 2 * px + (sub & 1);
-    } else {
-      ox = grow % p.Wo;
-      const int t = grow / p.Wo;
-      oy = t % p.Ho;
-      b = t / p.Ho;
-    }
-    return (b * p.PHs + oy * p.stride) * p.PWs + ox * p.stride;
-  };
+  // ---- tile geometry.  Only the tile's first row is decoded with full divisions (uniform); every
+  // other row and patch pixel is a small offset from it, for which the multiply-high quotients are
+  // exact. -----------------------------------------------------------------------------------------
   const int last_row = min(a0 + TA, p.rowsA) - 1;
   const int R = taps / p.S;
-  const int q_lo = row_base(a0);
-  const int q_hi = row_base(last_row) + (R - 1) * p.PWs + (p.S - 1);
+  const bool pooled = p.pool_order != 0;
+  const int gw = pooled ? p.Wo >> 1 : p.Wo, gh = pooled ? p.Ho >> 1 : p.Ho;  // row grid (windows when pooling)
+  const int gst = pooled ? 2 * p.stride : p.stride;                          // its step in the padded frame
+  const uint32_t u0 = (uint32_t)(pooled ? a0 >> 2 : a0);
+  const uint32_t t0 = u0 / (uint32_t)gw;
+  const int gx0 = (int)(u0 - t0 * (uint32_t)gw);
+  const int b0i = (int)(t0 / (uint32_t)gh);
+  const int gy0 = (int)(t0 - (uint32_t)b0i * (uint32_t)gh);
+  // padded-frame base index of tile row k (k >= 0, relative to a0), relative to the frame origin of image b0i
+  auto row_base = [&](int k) {
+    const int u = pooled ? k >> 2 : k, sub = pooled ? k & 3 : 0;
+    int gx = gx0 + u;
+    const int cy = (int)fast_div((uint32_t)gx, (uint32_t)gw, p.magicGW);
+    gx -= cy * gw;
+    int gy = gy0 + cy;
+    const int cb = (int)fast_div((uint32_t)gy, (uint32_t)gh, p.magicGH);
+    gy -= cb * gh;
+    return (cb * p.PHs + gy * gst + (sub >> 1) * p.stride) * p.PWs + gx * gst + (sub & 1) * p.stride;
+  };
+  const int q_lo = row_base(0);  // == (gy0*gst)*PWs + gx0*gst
+  const int q_hi = row_base(last_row - a0) + (R - 1) * p.PWs + (p.S - 1);
   const int npp = q_hi - q_lo + 1;
   if (npp > cap) return;  // the host sizes the patch for the worst tile; never taken
 
   // this lane's rows: patch-relative pixel index of row li of each of its FA row blocks
   int prow[FA];
 #pragma unroll
-  for (int x = 0; x < FA; ++x) prow[x] = row_base(min(a0 + (wa * FA + x) * 32 + li, last_row)) - q_lo;
+  for (int x = 0; x < FA; ++x) prow[x] = row_base(min((wa * FA + x) * 32 + li, last_row - a0)) - q_lo;
 
   // patch pixels this thread stages: global word offset of the pixel (channel word 0), or -1 for
   // padding / beyond the range
   long long poff[PATCH_NPT];
   const int pad_v = (p.PHs - p.Hs) >> 1;
-  const int frame = p.PHs * p.PWs;
+  const int yp0 = gy0 * gst, xp0 = gx0 * gst;
 #pragma unroll
   for (int j = 0; j < PATCH_NPT; ++j) {
     const int q = tid + j * NT;
     poff[j] = -1;
     if (q < npp) {
-      const int qq = q_lo + q;
-      const int img = qq / frame, rem = qq - img * frame;
-      const int yp = rem / p.PWs, xp = rem - yp * p.PWs;
+      int xp = xp0 + q;
+      const int cy = (int)fast_div((uint32_t)xp, (uint32_t)p.PWs, p.magicPW);
+      xp -= cy * p.PWs;
+      int yp = yp0 + cy;
+      const int ci = (int)fast_div((uint32_t)yp, (uint32_t)p.PHs, p.magicPH);
+      yp -= ci * p.PHs;
+      const int img = b0i + ci;
       const int iy = yp - pad_v, ix = xp - pad_v;
       if (img < p.batch && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws)
         poff[j] = (((long long)img * p.Hs + iy) * p.Ws + ix) * p.C32;
@@ -118,35 +125,83 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
   for (int cc = 0; cc < nchunks; ++cc) {
     const int cw = cc * 2;
     if (cc > 0) __syncthreads();  // every wave has finished reading the previous chunk
+    // ---- global loads of the chunk: patch pixels, then the first batch of filter tasks; all are in
+    // flight before the first one is consumed ----------------------------------------------------
+    uint32_t pw0[PATCH_NPT][PA], pw1[PATCH_NPT][PA];
+#pragma unroll
+    for (int j = 0; j < PATCH_NPT; ++j) {
+      const bool in = poff[j] >= 0;
+#pragma unroll
+      for (int pl = 0; pl < PA; ++pl) {
+        pw0[j][pl] = pw1[j][pl] = 0;
+        if (in) {
+          const uint32_t *src = p.A + pl * p.planeA + poff[j] + cw;
+          if (pair_ok) {
+            const uint2 v = *reinterpret_cast<const uint2 *>(src);
+            pw0[j][pl] = v.x;
+            pw1[j][pl] = v.y;
+          } else {
+            pw0[j][pl] = src[0];
+            if (cw + 1 < p.C32) pw1[j][pl] = src[1];
+          }
+        }
+      }
+    }
+    constexpr int FT = 4;  // filter tasks (tap, column) per thread and batch
+    const int ntask = taps * TB;
+    uint32_t fw0[FT][PB], fw1[FT][PB];
+    auto filter_load = [&](int first) {
+#pragma unroll
+      for (int j = 0; j < FT; ++j) {
+        const int t = first + tid + j * NT;
+        const int tap = t / TB, col = t % TB;
+        const int gcol = b0 + col;
+#pragma unroll
+        for (int pl = 0; pl < PB; ++pl) {
+          fw0[j][pl] = fw1[j][pl] = 0;
+          if (t < ntask && gcol < p.rowsB) {
+            const uint32_t *src = p.B + pl * p.planeB + ((long long)gcol * taps + tap) * p.C32 + cw;
+            if (pair_ok) {
+              const uint2 v = *reinterpret_cast<const uint2 *>(src);
+              fw0[j][pl] = v.x;
+              fw1[j][pl] = v.y;
+            } else {
+              fw0[j][pl] = src[0];
+              if (cw + 1 < p.C32) fw1[j][pl] = src[1];
+            }
+          }
+        }
+      }
+    };
+    auto filter_store = [&](int first) {
+#pragma unroll
+      for (int j = 0; j < FT; ++j) {
+        const int t = first + tid + j * NT;
+        if (t < ntask) {
+          const int tap = t / TB, col = t % TB;
+          static_for<0, DB>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            const v8i e0 = expand_fp4<PB, d>(fw0[j]), e1 = expand_fp4<PB, d>(fw1[j]);
+            uint4 *dst = reinterpret_cast<uint4 *>(filtB + (((d * taps + tap) * TB + col) * 2) * 4);
+            dst[0] = make_uint4((uint32_t)e0[0], (uint32_t)e0[1], (uint32_t)e0[2], (uint32_t)e0[3]);
+            dst[1] = make_uint4((uint32_t)e1[0], (uint32_t)e1[1], (uint32_t)e1[2], (uint32_t)e1[3]);
+          });
+        }
+      }
+    };
+    filter_load(0);
     // ---- patch chunk: packed words -> FP4 digit operands --------------------------------------
 #pragma unroll
     for (int j = 0; j < PATCH_NPT; ++j) {
       const int q = tid + j * NT;
       if (q < npp) {
-        uint32_t w0[PA], w1[PA];
-        const bool in = poff[j] >= 0;
-#pragma unroll
-        for (int pl = 0; pl < PA; ++pl) {
-          w0[pl] = w1[pl] = 0;
-          if (in) {
-            const uint32_t *src = p.A + pl * p.planeA + poff[j] + cw;
-            if (pair_ok) {
-              const uint2 v = *reinterpret_cast<const uint2 *>(src);
-              w0[pl] = v.x;
-              w1[pl] = v.y;
-            } else {
-              w0[pl] = src[0];
-              if (cw + 1 < p.C32) w1[pl] = src[1];
-            }
-          }
-        }
         int ps = 0;
 #pragma unroll
-        for (int pl = 0; pl < PA; ++pl) ps += (__popc(w0[pl]) + __popc(w1[pl])) << pl;
+        for (int pl = 0; pl < PA; ++pl) ps += (__popc(pw0[j][pl]) + __popc(pw1[j][pl])) << pl;
         pixsum[q] = ps;
         static_for<0, DA>([&](auto dc) {
           constexpr int d = decltype(dc)::value;
-          const v8i e0 = expand_fp4<PA, d>(w0), e1 = expand_fp4<PA, d>(w1);
+          const v8i e0 = expand_fp4<PA, d>(pw0[j]), e1 = expand_fp4<PA, d>(pw1[j]);
           uint4 *dst = reinterpret_cast<uint4 *>(patchA + ((d * cap + q) * 2) * 4);
           dst[0] = make_uint4((uint32_t)e0[0], (uint32_t)e0[1], (uint32_t)e0[2], (uint32_t)e0[3]);
           dst[1] = make_uint4((uint32_t)e1[0], (uint32_t)e1[1], (uint32_t)e1[2], (uint32_t)e1[3]);
@@ -154,32 +209,9 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
       }
     }
     // ---- filter chunk ----------------------------------------------------------------------
-    for (int t = tid; t < taps * TB; t += NT) {
-      const int tap = t / TB, col = t % TB;
-      const int gcol = b0 + col;
-      uint32_t w0[PB], w1[PB];
-#pragma unroll
-      for (int pl = 0; pl < PB; ++pl) {
-        w0[pl] = w1[pl] = 0;
-        if (gcol < p.rowsB) {
-          const uint32_t *src = p.B + pl * p.planeB + ((long long)gcol * taps + tap) * p.C32 + cw;
-          if (pair_ok) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(src);
-            w0[pl] = v.x;
-            w1[pl] = v.y;
-          } else {
-            w0[pl] = src[0];
-            if (cw + 1 < p.C32) w1[pl] = src[1];
-          }
-        }
-      }
-      static_for<0, DB>([&](auto dc) {
-        constexpr int d = decltype(dc)::value;
-        const v8i e0 = expand_fp4<PB, d>(w0), e1 = expand_fp4<PB, d>(w1);
-        uint4 *dst = reinterpret_cast<uint4 *>(filtB + (((d * taps + tap) * TB + col) * 2) * 4);
-        dst[0] = make_uint4((uint32_t)e0[0], (uint32_t)e0[1], (uint32_t)e0[2], (uint32_t)e0[3]);
-        dst[1] = make_uint4((uint32_t)e1[0], (uint32_t)e1[1], (uint32_t)e1[2], (uint32_t)e1[3]);
-      });
+    for (int first = 0; first < ntask; first += FT * NT) {
+      filter_store(first);
+      if (first + FT * NT < ntask) filter_load(first + FT * NT);
     }
     __syncthreads();
 
