@@ -197,5 +197,6 @@ class Network {
 
 std::unique_ptr<Network> build_alexnet(int batch, uint64_t seed, int path);
 std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path);
+std::unique_ptr<Network> build_vgg(int batch, uint64_t seed, int path);
 
 }  // namespace apnn_nn

@@ -56,6 +56,41 @@ std::unique_ptr<Network> build_alexnet(int batch, uint64_t seed, int path) {
   return net;
 }
 
+// VGG-variant of APNN-TC-nn/src/vgg.cu:49-127: ten 3x3 convolutions (3->96 stride 2, 96->256, 256->256 x2,
+// 256->512, 512->512 x5) with 2x2 pooling after the 1st, 4th, 7th and 10th, FC 4096 x2, 1000 outputs.
+// The first convolution runs in int8 on the raw image (the reference quantizes the image to bit-planes
+// instead, vgg.cu:46-52).
+std::unique_ptr<Network> build_vgg(int batch, uint64_t seed, int path) {
+  auto net = std::make_unique<Network>();
+  net->batch = batch;
+  Rng rng(seed);
+  auto *c1 = add(*net, new InConv128LayerParam("Conv1", 224, 224, 3, 3, 3, 96, batch, 2, 2, true, 2, 2));
+  if (c1->initialize(rng, nullptr)) return nullptr;
+  net->first = c1;
+  const int chans[9] = {256, 256, 256, 512, 512, 512, 512, 512, 512};
+  const uint32_t *prev = c1->get_output_gpu();
+  int h = c1->output_height, w = c1->output_width, cin = 96;
+  for (int i = 0; i < 9; ++i) {
+    char nm[16];
+    snprintf(nm, sizeof nm, "Conv%d", i + 2);
+    const int pool = (i == 2 || i == 5 || i == 8) ? 2 : 1;  // Conv4, Conv7, Conv10
+    auto *c = add(*net, new Conv128LayerParam(nm, h, w, 3, 3, cin, chans[i], batch, 1, 1, true, pool, pool));
+    if (c->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+    prev = c->get_output_gpu();
+    h = c->output_height;
+    w = c->output_width;
+    cin = chans[i];
+  }
+  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, h, w, 512, 4096));
+  if (f1->initialize(rng, prev, path)) return nullptr;
+  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 1, 1, 4096, 4096));
+  if (f2->initialize(rng, f1->get_output_gpu(), path)) return nullptr;
+  auto *out = add(*net, new Out128LayerParam("Fout", batch, 1, 4096, 1000, -1));
+  if (out->initialize(rng, f2->get_output_gpu(), nullptr)) return nullptr;
+  net->last = out;
+  return net;
+}
+
 // Standard ResNet18: 7x7/2 int8 stem + 3x3/2 max-pool, four stages of two basic blocks at
 // 64/128/256/512 channels, a strided 1x1 convolution on the shortcut where the shape changes, global
 // average pool and an int8 classifier.  (The reference's own demo, APNN-TC-nn/src/resnet18.cu:40-142,
@@ -120,6 +155,8 @@ apnn_net *apnn_net_create(int kind, int batch, unsigned long long seed, int path
     n = apnn_nn::build_alexnet(batch, seed, path);
   } else if (kind == APNN_NET_RESNET18) {
     n = apnn_nn::build_resnet18(batch, seed, path);
+  } else if (kind == APNN_NET_VGG) {
+    n = apnn_nn::build_vgg(batch, seed, path);
   }
   if (!n) return nullptr;
   apnn_net *h = new (std::nothrow) apnn_net;

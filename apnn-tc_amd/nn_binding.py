@@ -4,11 +4,11 @@ import os
 
 from . import binding
 
-__all__ = ["NN_LIB_PATH", "nn_lib", "LayerDesc", "NET_ALEXNET", "NET_RESNET18",
+__all__ = ["NN_LIB_PATH", "nn_lib", "LayerDesc", "NET_ALEXNET", "NET_RESNET18", "NET_VGG",
            "LAYER_INCONV_I8", "LAYER_CONV", "LAYER_FC", "LAYER_OUT_I8", "NN_DECLARED_SYMBOLS"]
 
 NN_LIB_PATH = os.path.join(binding.PKG_DIR, "lib", "libapnn_nn.so")
-NET_ALEXNET, NET_RESNET18 = 0, 1
+NET_ALEXNET, NET_RESNET18, NET_VGG = 0, 1, 2
 LAYER_INCONV_I8, LAYER_CONV, LAYER_FC, LAYER_OUT_I8 = 0, 1, 2, 3
 NN_DECLARED_SYMBOLS = ["apnn_net_create", "apnn_net_destroy", "apnn_net_forward", "apnn_net_forward_graph",
                        "apnn_net_layer_count", "apnn_net_layer", "apnn_net_bench", "apnn_nn_download"]

@@ -46,7 +46,7 @@ def main():
     ap.add_argument("--extra", default="all",
                     help="comma list of secondary workloads to run after the headline: all, none, gemm_sweep, "
                          "gemm_large, gemm8192 (w1a2 only), conv, nets, resnet18_b8, resnet18_b64, alexnet_b8, "
-                         "alexnet_b64")
+                         "alexnet_b64, vgg_b8, vgg_b64")
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one 256 MiB device copy (known traffic) for counter calibration")
@@ -220,7 +220,7 @@ def main():
             extra["conv"] = convs
         # ---- second headline metric: end-to-end w1a2 ResNet18 (and the AlexNet-style net) --------
         nets = {}
-        for kind, nm in ((A.NET_RESNET18, "resnet18"), (A.NET_ALEXNET, "alexnet")):
+        for kind, nm in ((A.NET_RESNET18, "resnet18"), (A.NET_ALEXNET, "alexnet"), (A.NET_VGG, "vgg")):
             for batch in (8, 64):
                 if not on("nets", "%s_b%d" % (nm, batch)):
                     continue

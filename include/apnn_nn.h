@@ -20,7 +20,9 @@ extern "C" {
 #endif
 
 enum { APNN_NET_ALEXNET = 0,   /* topology of APNN-TC-nn/src/alexnet.cu:42-81, int8 first conv / classifier */
-       APNN_NET_RESNET18 = 1 };/* standard ResNet18 (3x3 basic blocks, strided 1x1 downsample convs)        */
+       APNN_NET_RESNET18 = 1,  /* standard ResNet18 (3x3 basic blocks, strided 1x1 downsample convs)        */
+       APNN_NET_VGG = 2 };     /* topology of APNN-TC-nn/src/vgg.cu:49-127 (ten 3x3 convs, 96..512 channels,
+                                  first one stride 2; 2x2 pools after convs 1, 4, 7, 10; two 4096 FCs)       */
 
 enum { APNN_LAYER_INCONV_I8 = 0, /* int8 conv + thresholds (+ max-pool) + pack                               */
        APNN_LAYER_CONV = 1,      /* low-bit conv, fused threshold / pool / shortcut epilogue                  */

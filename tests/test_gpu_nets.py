@@ -129,3 +129,9 @@ def test_alexnet_layer_by_layer(G, path):
 
 def test_resnet18_graph_replay(G):
     _check_network(G, G.A.NET_RESNET18, 2, 0, graph=True)
+
+
+@pytest.mark.parametrize("path", [0, 2])
+def test_vgg_layer_by_layer(G, path):
+    n = _check_network(G, G.A.NET_VGG, 2, path, graph=False)
+    assert n == 10 + 2 + 1          # ten convolutions, two hidden FCs, classifier
