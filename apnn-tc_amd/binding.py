@@ -44,9 +44,10 @@ class ConvDesc(ctypes.Structure):
 _GEMM_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp]
 _CONV_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 
-_GEMM_NAMES = ["apmm_w1a2", "apmm_w1a3", "apmm_w1a4", "apmm_w2a2",
+_GEMM_NAMES = ["apmm_w1a2", "apmm_w1a3", "apmm_w1a4", "apmm_w2a2", "apmm_w1a8", "apmm_w2a8", "apmm_w4a4", "apmm_w1a1",
                "apmm_w1a2_decompose", "apmm_w1a3_decompose", "apmm_w1a4_decompose", "apmm_w2a2_decompose"]
-_CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2",
+_CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2", "apconv_w1a5", "apconv_w2a6",
+               "APConv_w2a8_pack",
                "APConv_w1a2_pack", "APConv_w1a3_pack", "APConv_w1a4_pack", "APConv_w2a2_pack",
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
 DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",

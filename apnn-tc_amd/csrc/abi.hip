@@ -240,7 +240,7 @@ valu_fn valu_gemm_fn(int wb, int xb) {
   if (wb == 1 && xb == 3) return apnn::valu_gemm_1_3_x;
   if (wb == 1 && xb == 4) return apnn::valu_gemm_1_4_x;
   if (wb == 2 && xb == 2) return apnn::valu_gemm_2_2_x;
-  return nullptr;
+  return apnn::valu_gemm_any_x;  // 1..8 planes each, one 32x32-tile kernel
 }
 
 valu_fn valu_conv_fn(int xb, int wb) {
@@ -248,7 +248,7 @@ valu_fn valu_conv_fn(int xb, int wb) {
   if (xb == 3 && wb == 1) return apnn::valu_conv_3_1_x;
   if (xb == 4 && wb == 1) return apnn::valu_conv_4_1_x;
   if (xb == 2 && wb == 2) return apnn::valu_conv_2_2_x;
-  return nullptr;
+  return apnn::valu_conv_any_x;
 }
 
 int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
@@ -259,7 +259,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
-  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_I8))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_PATCH))
     return APNN_EINVAL;
   if ((rc = check_epilogue(d->epi, d->N, false, 0, 0))) return rc;
 
@@ -276,12 +276,16 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->D, d->M);
 
   int tile;
+  p.planesA = d->wb;
+  p.planesB = d->xb;
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
-    if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, false, 4, path == APNN_PATH_MFMA_I8, &tile))) return rc;
-    return from_hip(fn(4, tile, p, stream));
+    if (fn != nullptr) {
+      if ((rc = pick_mfma_tile(tile_pin, p, false, 4, path == APNN_PATH_MFMA_I8, &tile))) return rc;
+      return from_hip(fn(4, tile, p, stream));
+    }
+    if (path != APNN_PATH_AUTO) return APNN_EUNSUPPORTED;  // precisions without a matrix-core kernel
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
@@ -336,6 +340,8 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
 
   int tile;
+  p.planesA = d->xb;
+  p.planesB = d->wb;
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;
@@ -354,9 +360,11 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   }
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
     valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
-    if (fn == nullptr) return APNN_EUNSUPPORTED;
-    if ((rc = pick_mfma_tile(tile_pin, p, true, vw, false, &tile))) return rc;
-    return from_hip(fn(vw, tile, p, stream));
+    if (fn != nullptr) {
+      if ((rc = pick_mfma_tile(tile_pin, p, true, vw, false, &tile))) return rc;
+      return from_hip(fn(vw, tile, p, stream));
+    }
+    if (path != APNN_PATH_AUTO) return APNN_EUNSUPPORTED;
   }
   valu_fn fn = valu_conv_fn(d->xb, d->wb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
@@ -422,6 +430,10 @@ APNN_DEF_GEMM(apmm_w1a2, 1, 2, APNN_EPI_INT32)
 APNN_DEF_GEMM(apmm_w1a3, 1, 3, APNN_EPI_INT32)
 APNN_DEF_GEMM(apmm_w1a4, 1, 4, APNN_EPI_INT32)
 APNN_DEF_GEMM(apmm_w2a2, 2, 2, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w1a8, 1, 8, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w2a8, 2, 8, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w4a4, 4, 4, APNN_EPI_INT32)
+APNN_DEF_GEMM(apmm_w1a1, 1, 1, APNN_EPI_INT32)
 APNN_DEF_GEMM(apmm_w1a2_decompose, 1, 2, APNN_EPI_LOWBITS)
 APNN_DEF_GEMM(apmm_w1a3_decompose, 1, 3, APNN_EPI_LOWBITS)
 APNN_DEF_GEMM(apmm_w1a4_decompose, 1, 4, APNN_EPI_LOWBITS)
@@ -437,6 +449,9 @@ APNN_DEF_CONV(apconv_w1a2, 1, 2, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w1a3, 1, 3, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w1a4, 1, 4, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w2a2, 2, 2, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w1a5, 1, 5, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w2a6, 2, 6, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w2a8_pack, 2, 8, APNN_EPI_LOWBITS, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w1a2_pack, 1, 2, APNN_EPI_LOWBITS, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w1a3_pack, 1, 3, APNN_EPI_LOWBITS, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w1a4_pack, 1, 4, APNN_EPI_LOWBITS, APNN_POOL_NONE)

@@ -17,6 +17,8 @@ APNN_DECL_VALU(conv, 3, 1)
 APNN_DECL_VALU(conv, 4, 1)
 APNN_DECL_VALU(conv, 2, 2)
 #undef APNN_DECL_VALU
+hipError_t valu_gemm_any_x(int vw, int tile, const KParams &p, hipStream_t s);
+hipError_t valu_conv_any_x(int vw, int tile, const KParams &p, hipStream_t s);
 
 #define APNN_DECL_MFMA(kind, pa, pb) \
   hipError_t mfma_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);

@@ -16,6 +16,7 @@ struct KParams {
   const uint32_t *B;
   int rowsA, rowsB;          // logical output size out[rowsA][rowsB]
   int KW;                    // reduction length in 32-bit words (GEMM: K/32, conv: R*S*C32)
+  int planesA, planesB;      // bit-planes of A / B (read by the any-precision kernel instantiation only)
   long long planeA, planeB;  // plane strides in words
 
   // implicit im2col (convolution kernels only); halo-stored inputs are expressed as pad = 0 on the

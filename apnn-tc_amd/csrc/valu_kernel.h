@@ -50,6 +50,10 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t d, uint32_t m)
 
 template <int PA, int PB, int RA, int RB, int VW, bool CONV>
 __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
+  // PA == PB == 8 is the any-precision instantiation: the plane counts of the launch (1..8 each) come
+  // from KParams and the plane loops skip what is not there.
+  constexpr bool ANY = PA == 8 && PB == 8;
+  const int na = ANY ? p.planesA : PA, nb = ANY ? p.planesB : PB;
   constexpr int NT = 256;
   constexpr int TA = 16 * RA, TB = 16 * RB;
   constexpr int KC = 16;            // k-words per staged chunk
@@ -152,7 +156,8 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
         off = (long long)(a0 + a_row[it]) * p.KW + kw0;
       }
 #pragma unroll
-      for (int pl = 0; pl < PA; ++pl) load_words<VW>(p.A + off + pl * p.planeA, ok, ra_[it][pl]);
+      for (int pl = 0; pl < PA; ++pl)
+        if (!ANY || pl < na) load_words<VW>(p.A + off + pl * p.planeA, ok, ra_[it][pl]);
     }
 #pragma unroll
     for (int it = 0; it < NIB; ++it) {
@@ -160,7 +165,8 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
       const bool ok = b_ok[it] && kw0 < p.KW;
       const long long off = (long long)(b0 + b_row[it]) * p.KW + kw0;
 #pragma unroll
-      for (int pl = 0; pl < PB; ++pl) load_words<VW>(p.B + off + pl * p.planeB, ok, rb_[it][pl]);
+      for (int pl = 0; pl < PB; ++pl)
+        if (!ANY || pl < nb) load_words<VW>(p.B + off + pl * p.planeB, ok, rb_[it][pl]);
     }
   };
 
@@ -170,8 +176,10 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
       if (UA % NT == 0 || tid + it * NT < UA) {
 #pragma unroll
         for (int pl = 0; pl < PA; ++pl)
+          if (!ANY || pl < na) {
 #pragma unroll
-          for (int i = 0; i < VW; ++i) As[(pl * KC + a_kq[it] * VW + i) * LDA + a_row[it]] = ra_[it][pl][i];
+            for (int i = 0; i < VW; ++i) As[(pl * KC + a_kq[it] * VW + i) * LDA + a_row[it]] = ra_[it][pl][i];
+          }
       }
     }
 #pragma unroll
@@ -179,8 +187,10 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
       if (UB % NT == 0 || tid + it * NT < UB) {
 #pragma unroll
         for (int pl = 0; pl < PB; ++pl)
+          if (!ANY || pl < nb) {
 #pragma unroll
-          for (int i = 0; i < VW; ++i) Bs[(pl * KC + b_kq[it] * VW + i) * LDB + b_row[it]] = rb_[it][pl][i];
+            for (int i = 0; i < VW; ++i) Bs[(pl * KC + b_kq[it] * VW + i) * LDB + b_row[it]] = rb_[it][pl][i];
+          }
       }
     }
   };
@@ -211,17 +221,33 @@ __global__ __launch_bounds__(256) void apnn_valu_kernel(const KParams p) {
     for (int kw = 0; kw < KC; ++kw) {
       uint32_t a[PA][RA], b[PB][RB];
 #pragma unroll
-      for (int pl = 0; pl < PA; ++pl) lds_read_rows<RA>(&As[(pl * KC + kw) * LDA + ta * RA], a[pl]);
+      for (int pl = 0; pl < PA; ++pl) {
+        if (!ANY || pl < na) {
+          lds_read_rows<RA>(&As[(pl * KC + kw) * LDA + ta * RA], a[pl]);
+        } else {
 #pragma unroll
-      for (int pl = 0; pl < PB; ++pl) lds_read_rows<RB>(&Bs[(pl * KC + kw) * LDB + tb * RB], b[pl]);
+          for (int x = 0; x < RA; ++x) a[pl][x] = 0;
+        }
+      }
+#pragma unroll
+      for (int pl = 0; pl < PB; ++pl) {
+        if (!ANY || pl < nb) {
+          lds_read_rows<RB>(&Bs[(pl * KC + kw) * LDB + tb * RB], b[pl]);
+        } else {
+#pragma unroll
+          for (int y = 0; y < RB; ++y) b[pl][y] = 0;
+        }
+      }
 #pragma unroll
       for (int i = 0; i < PA; ++i)
 #pragma unroll
         for (int j = 0; j < PB; ++j)
+          if (!ANY || (i < na && j < nb)) {
 #pragma unroll
-          for (int x = 0; x < RA; ++x)
+            for (int x = 0; x < RA; ++x)
 #pragma unroll
-            for (int y = 0; y < RB; ++y) acc[i + j][x][y] += __popc(a[i][x] & b[j][y]);
+              for (int y = 0; y < RB; ++y) acc[i + j][x][y] += __popc(a[i][x] & b[j][y]);
+          }
       if (p.sym) {
 #pragma unroll
         for (int i = 0; i < PS; ++i)
@@ -308,6 +334,12 @@ inline hipError_t launch_valu_tile(int tile, const KParams &p, hipStream_t strea
     case TILE_16x32: return launch_valu<PA, PB, 1, 2, VW, CONV>(p, stream);
     default: return launch_valu<PA, PB, 1, 1, VW, CONV>(p, stream);
   }
+}
+
+// any-precision instantiation: 32x32 tile only
+template <int VW, bool CONV>
+inline hipError_t launch_valu_any(const KParams &p, hipStream_t stream) {
+  return launch_valu<8, 8, 2, 2, VW, CONV>(p, stream);
 }
 
 }  // namespace apnn

@@ -48,6 +48,15 @@ int apmm_w1a3(const void *W, const void *X, int *D, int M, int N, int K, int wb,
 int apmm_w1a4(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
 int apmm_w2a2(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
 
+/* Further precisions of the reference tree, same definition and constraints: apmm_w1a8
+ * (LIB/77_bmmaTensorCoreGemm.cu:80), apmm_w2a8 (LIB/76_bmmaTensorCoreGemm.cuh:80-82), apmm_w4a4
+ * (LIB/83_bmmaTensorCoreGemm.cu:80), apmm_w1a1 (LIB/84_bmmaTensorCoreGemm.cu:80).  Any other (w, a) up to
+ * 8 bits each is served by apnn_gemm / apnn_conv.  These run on the any-precision VALU kernel. */
+int apmm_w1a8(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w2a8(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w4a4(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+int apmm_w1a1(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
+
 /* Same accumulate, then the low xb bits of each result packed MSB-first along N:
  * D:[xb][M][N/32] uint32.  Replace apmm_w1a2_decompose (LIB/66h:82-280) and apmm_w2a2_decompose
  * (LIB/73_bmmaTensorCoreGemm.cuh:82).  Requires N % 32 == 0. */
@@ -65,6 +74,10 @@ int apconv_w1a3(const void *W, const void *X, int *Output, int Height, int Width
 int apconv_w1a4(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 int apconv_w2a2(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 
+/* compute_conv_imma at w1a5 (LIB/61_bmmaTensorCoreGemm.cu:58, LIB/62) and w2a6 (LIB/63_bmmaTensorCoreGemm.cu:58). */
+int apconv_w1a5(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int apconv_w2a6(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+
 /* Convolution, then low-bit planes of the result: Output:[a][H][W][COUT/32].
  * Replace APConv_w1a2_pack (LIB/67h:60-325) and APConv_w2a2_pack (LIB/70_bmmaTensorCoreGemm.cu:58).
  * Requires COUT % 32 == 0. */
@@ -72,6 +85,9 @@ int APConv_w1a2_pack(const void *W, const void *X, int *Output, int Height, int 
 int APConv_w1a3_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 int APConv_w1a4_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 int APConv_w2a2_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+
+/* APConv_w2a8_pack (LIB/74_bmmaTensorCoreGemm.cuh:58-61): Output:[8][H][W][COUT/32]. */
+int APConv_w2a8_pack(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 
 /* Convolution, 2x2 average pool with C integer division, then low-bit planes:
  * Output:[a][H/2][W/2][COUT/32].  Replace APConv_w1a2_pack_pool (LIB/68_bmmaTensorCoreGemm.cu:58)

@@ -100,7 +100,11 @@ def test_combinations_that_are_not_built_are_reported():
     assert L.apnn_conv(ctypes.byref(c), None) == A.EUNSUPPORTED          # int8 core: GEMM entry points only
     g = A.GemmDesc(W=good, X=good, D=good, M=64, N=128, K=128, wb=1, xb=2, path=A.PATH_MFMA | (1 << 8))
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # FP4 GEMM has no 256x256 tile
-    g.wb, g.xb, g.path = 3, 5, A.PATH_AUTO
-    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # only w1a2 / w1a3 / w1a4 / w2a2 are built
+    g.wb, g.xb, g.path = 3, 5, A.PATH_MFMA
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # matrix-core kernels: w1a2 / w1a3 / w1a4 / w2a2
+    g.path = A.PATH_MFMA_PATCH
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # convolution only
+    g.wb, g.xb, g.path = 9, 2, A.PATH_AUTO
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL                # at most 8 planes per operand
     g.wb, g.xb, g.path = 1, 2, A.PATH_VALU | (9 << 8)
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL                # no such tile

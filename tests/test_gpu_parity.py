@@ -535,3 +535,72 @@ def test_gemm_quantize_pack_all_widths(G, path, tile, wb, xb, ob, sym):
     q = O.bn_quantize(acc, None, thr, flip, ob)
     assert 0 < q.mean() < 2 ** ob - 1
     assert np.array_equal(got, O.lowbits_pack(q, M, N, ob))
+
+
+# ---- further precisions of the reference tree (any-precision kernel) -------------------------------
+@pytest.mark.parametrize("wb,xb", [(1, 8), (2, 8), (4, 4), (1, 1)])
+def test_gemm_named_entry_more_precisions(G, wb, xb):
+    rng = np.random.default_rng(5000 + 10 * wb + xb)
+    M, N, K = 64, 96, 256
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    dW, dX, out = G.to_dev(W), G.to_dev(X), G.dev_empty_i32(M * N, fill=-7)
+    fn = getattr(G.A.lib(), "apmm_w%da%d" % (wb, xb))
+    G.A.check(fn(G.ptr(dW), G.ptr(dX), G.ptr(out), M, N, K, wb, xb, None), "apmm")
+    got = G.to_host(out).reshape(M, N)
+    assert np.array_equal(got, O.unpack_planes_lsb(W) @ O.unpack_planes_lsb(X).T)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb))
+    # wrong bit widths for the name are rejected
+    assert fn(G.ptr(dW), G.ptr(dX), G.ptr(out), M, N, K, wb + 1, xb, None) == G.A.EINVAL
+
+
+@pytest.mark.parametrize("name,wb,xb,pack", [("apconv_w1a5", 1, 5, False), ("apconv_w2a6", 2, 6, False),
+                                             ("APConv_w2a8_pack", 2, 8, True)])
+def test_conv_named_entry_more_precisions(G, name, wb, xb, pack):
+    rng = np.random.default_rng(5100 + 10 * wb + xb)
+    H, Wd, C, cout = 6, 8, 128, 64
+    X = O.random_planes(rng, xb, (H + 2) * (Wd + 2), C // 32)
+    Xv = X.reshape(xb, H + 2, Wd + 2, C // 32)
+    Xv[:, 0], Xv[:, -1], Xv[:, :, 0], Xv[:, :, -1] = 0, 0, 0, 0
+    Wt = O.random_planes(rng, wb, cout * 9, C // 32)
+    kw = dict(batch=1, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=1, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, **kw)
+    dW, dX = G.to_dev(Wt), G.to_dev(X)
+    words = xb * H * Wd * cout // 32 if pack else H * Wd * cout
+    out = G.dev_empty_i32(words, fill=-7)
+    G.A.check(getattr(G.A.lib(), name)(G.ptr(dW), G.ptr(dX), G.ptr(out), H, Wd, C, cout, None), name)
+    if pack:
+        expect = O.lowbits_pack(acc.reshape(-1, cout), H * Wd, cout, xb)
+        assert np.array_equal(G.to_host(out, np.uint32).reshape(expect.shape), expect)
+    else:
+        assert np.array_equal(G.to_host(out).reshape(acc.shape), acc)
+
+
+@pytest.mark.parametrize("wb,xb,ob", [(3, 5, 4), (8, 8, 2), (1, 7, 3), (5, 1, 1)])
+@pytest.mark.parametrize("sym", [0, 1])
+def test_any_precision_descriptor_paths(G, wb, xb, ob, sym):
+    """apnn_gemm / apnn_conv at bit widths without a dedicated kernel: AUTO and the VALU path serve
+    them (bit-exact, all epilogues), the matrix-core paths report APNN_EUNSUPPORTED."""
+    rng = np.random.default_rng(5200 + 100 * wb + 10 * xb + sym)
+    M, N, K = 40, 64, 128
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, wb, xb, sym_w=sym)
+    for path in (0, 1):
+        assert np.array_equal(G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=path).reshape(M, N), acc)
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):
+        G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=2)
+    thr = np.sort(rng.integers(int(acc.min()), int(acc.max()) + 1, size=(N, 2 ** ob - 1)), axis=1).astype(np.int32)
+    d_thr = G.to_dev(thr)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, epi=epi).view(np.uint32).reshape(ob, M, N // 32)
+    assert np.array_equal(got, O.lowbits_pack(O.bn_quantize(acc, None, thr, None, ob), M, N, ob))
+    # convolution, stride 2, 32 stored channels
+    batch, H, Wd, C, cout = 2, 9, 7, 32, 40
+    Xc = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wc = O.random_planes(rng, wb, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=2, pad=1, halo=0, wb=wb, xb=xb)
+    expect = O.conv(Wc, Xc, cwords=C // 32, sym_w=sym, **kw)
+    assert np.array_equal(G.run_conv(Wc, Xc, cin_pad=C, sym=sym, **kw).reshape(expect.shape), expect)
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):
+        G.run_conv(Wc, Xc, cin_pad=C, sym=sym, path=4, **kw)
