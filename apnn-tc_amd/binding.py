@@ -52,7 +52,7 @@ _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2", "apco
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
 DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
                                                 "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
-                                                "apnn_conv_i8_bn_pack", "apnn_pool_planes",
+                                                "apnn_conv_i8_bn_pack", "apnn_pool_planes", "apnn_quantize_pack", "apnn_fold_bn",
                                                 "apnn_device_cus", "apnn_version"]
 
 
@@ -116,6 +116,10 @@ def lib():
         L.apnn_unpack_sum.restype = _ci
         L.apnn_fc_i8.argtypes = [_vp] * 6 + [_ci] * 3 + [_vp]
         L.apnn_fc_i8.restype = _ci
+        L.apnn_quantize_pack.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, ctypes.c_float, ctypes.c_float, _vp]
+        L.apnn_quantize_pack.restype = _ci
+        L.apnn_fold_bn.argtypes = [_vp] * 4 + [ctypes.c_float] * 3 + [_ci, _ci, _vp, _vp]
+        L.apnn_fold_bn.restype = _ci
         L.apnn_device_cus.argtypes = []
         L.apnn_device_cus.restype = _ci
         L.apnn_version.argtypes = []

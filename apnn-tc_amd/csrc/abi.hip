@@ -1,6 +1,9 @@
 // C ABI: argument validation, kernel-path / tile selection and launch.  See include/apnn_tc.h.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
+#include <cstdint>
+
 #include <atomic>
 
 #include "../../include/apnn_tc.h"
@@ -468,6 +471,51 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
   if (values == nullptr || planes == nullptr) return APNN_ENULL;
   if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 32) return APNN_EINVAL;
   return (int)apnn::launch_pack_bits(values, planes, rows, C, cpad, bits, static_cast<hipStream_t>(s));
+}
+
+int apnn_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
+                       float max_v, apnn_stream_t s) {
+  if (values == nullptr || planes == nullptr) return APNN_ENULL;
+  if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 16 || !(max_v > min_v))
+    return APNN_EINVAL;
+  return (int)apnn::launch_quantize_pack(values, planes, rows, C, cpad, bits, min_v, max_v,
+                                         static_cast<hipStream_t>(s));
+}
+
+int apnn_fold_bn(const float *gamma, const float *beta, const float *mean, const float *var, float eps,
+                 float in_scale, float step, int C, int bits, int32_t *thresholds, uint8_t *flip) {
+  if (gamma == nullptr || beta == nullptr || mean == nullptr || var == nullptr || thresholds == nullptr ||
+      flip == nullptr)
+    return APNN_ENULL;
+  if (C <= 0 || bits < 1 || bits > 8 || !(step > 0.0f) || in_scale == 0.0f) return APNN_EINVAL;
+  const int nt = (1 << bits) - 1;
+  const double lo = -2147483648.0, hi = 2147483647.0;
+  for (int c = 0; c < C; ++c) {
+    const double denom = std::sqrt((double)var[c] + (double)eps);
+    if (!(denom > 0.0)) return APNN_EINVAL;
+    const double slope = (double)gamma[c] / denom;          // dy / d(v * in_scale)
+    const double dir = slope * (double)in_scale;            // dy / dv
+    auto y_of = [&](double v) { return slope * (v * (double)in_scale - (double)mean[c]) + (double)beta[c]; };
+    int32_t *t = thresholds + (long long)c * nt;
+    flip[c] = dir < 0.0 ? 1 : 0;
+    for (int k = 1; k <= nt; ++k) {
+      const double target = (double)k * (double)step;
+      if (dir == 0.0) {  // constant output: the comparison is always / never true
+        t[k - 1] = (double)beta[c] >= target ? INT32_MIN : INT32_MAX;
+        continue;
+      }
+      // u = v (rising) or -v (falling): smallest integer u with y >= target
+      const double sgn = dir < 0.0 ? -1.0 : 1.0;
+      double u = std::ceil(sgn * ((target - (double)beta[c]) / slope + (double)mean[c]) / (double)in_scale);
+      if (u < lo) u = lo;
+      if (u > hi) u = hi;
+      // make the closed form agree with y_of() itself at the boundary
+      for (int it = 0; it < 4 && u > lo && y_of(sgn * (u - 1.0)) >= target; ++it) u -= 1.0;
+      for (int it = 0; it < 4 && u < hi && !(y_of(sgn * u) >= target); ++it) u += 1.0;
+      t[k - 1] = (int32_t)u;
+    }
+  }
+  return APNN_OK;
 }
 
 int apnn_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thresholds, uint8_t *codes, int32_t *acc_out,

@@ -29,6 +29,48 @@ __global__ __launch_bounds__(256) void pack_bits_kernel(const uint32_t *__restri
   }
 }
 
+// Quantize_val (APNN-TC-nn/src/kernel.cuh:29-44) fused with the packer above: float -> code -> planes.
+__global__ __launch_bounds__(256) void quantize_pack_kernel(const float *__restrict__ values,
+                                                            uint32_t *__restrict__ planes, int rows, int C,
+                                                            int cpad, int bits, float min_v, float max_v) {
+  const int lane = threadIdx.x & 63;
+  const int wave_in_block = threadIdx.x >> 6;
+  const int cw = cpad >> 5;
+  const int groups = (cpad + 63) >> 6;
+  const long long total = (long long)rows * groups;
+  const long long plane_stride = (long long)rows * cw;
+  const uint32_t top = (1u << bits) - 1u;
+  const float levels = (float)(1 << bits), range = max_v - min_v;
+  for (long long g = (long long)blockIdx.x * 4 + wave_in_block; g < total; g += (long long)gridDim.x * 4) {
+    const int row = (int)(g / groups);
+    const int c = (int)(g % groups) * 64 + lane;
+    uint32_t v = 0u;
+    if (c < C) {
+      float x = values[(long long)row * C + c];
+      x = x < min_v ? min_v : (x > max_v ? max_v : x);
+      const float q = __fdiv_rn(__fmul_rn(__fmul_rn(__fsub_rn(x, min_v), levels), 1.0f), range);
+      v = min(top, __float2uint_rn(q));
+    }
+    for (int b = 0; b < bits; ++b) {
+      const unsigned long long mask = __ballot((v >> b) & 1u);
+      const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
+      const int wi = c >> 5;
+      if ((lane & 31) == 0 && wi < cw) planes[b * plane_stride + (long long)row * cw + wi] = word;
+    }
+  }
+}
+
+hipError_t launch_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
+                                float max_v, hipStream_t s) {
+  const long long total = (long long)rows * ((cpad + 63) / 64);
+  long long blocks = (total + 3) / 4;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(quantize_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, values, planes, rows, C, cpad, bits,
+                     min_v, max_v);
+  return hipGetLastError();
+}
+
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
                             hipStream_t s) {
   const long long total = (long long)rows * ((cpad + 63) / 64);

@@ -59,6 +59,9 @@ constexpr int kPatchTileCols[kPatchTileCount] = {128, 64, 128, 64, 64};
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
                             hipStream_t s);
 
+hipError_t launch_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
+                                float max_v, hipStream_t s);
+
 // nn_kernels.hip
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
                              uint32_t *planes, int B, int H, int W, int C, int COUT, int R, int S, int stride, int pad,

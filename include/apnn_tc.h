@@ -179,6 +179,24 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
 
 /* ---- layers on either side of the low-bit path ------------------------------------------------ */
 
+/* Float tensor -> bit-planes in one pass: the affine quantizer of Quantize_val
+ * (APNN-TC-nn/src/kernel.cuh:29-44; the reference computes the code but its store is commented out)
+ *     code = min(2^bits - 1, rint(((clip(x, min_v, max_v) - min_v) * 2^bits * 1.0f) / (max_v - min_v)))
+ * in fp32 with exactly that operation order (rint = round half to even, __float2uint_rn), followed by
+ * the Bit_compression layout of apnn_pack_bits.  values:[rows][C] float; planes:[bits][rows][cpad/32].
+ * The reference fixes min_v = -10, max_v = 10 (kernel.cuh:17-18). */
+int apnn_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
+                       float max_v, apnn_stream_t s);
+
+/* Host-side preparation (no device work): fold a batch-norm + uniform activation quantizer into the
+ * integer thresholds of APNN_EPI_BN.  With y(v) = gamma[c] * (v * in_scale - mean[c]) / sqrt(var[c] + eps)
+ * + beta[c] evaluated in double precision, code = clamp(floor(y / step), 0, 2^bits - 1) equals
+ * #{k : s_c * v >= thresholds[c][k]} for every int32 v, where flip[c] = 1 (s_c = -1) when y decreases in
+ * v.  thresholds:[C][2^bits-1] int32 (host), flip:[C] bytes (host).  The reference folds only a 1-bit
+ * threshold offline (its layers read one float per channel, APNN-TC-nn/src/kernel.cuh:833-834). */
+int apnn_fold_bn(const float *gamma, const float *beta, const float *mean, const float *var, float eps,
+                 float in_scale, float step, int C, int bits, int32_t *thresholds, uint8_t *flip);
+
 /* int8 NHWC convolution with zero padding (the first layer of a network, cf. the int8 convention of
  * cutlass_nn/src/config.h:215-255: int8 operands, int32 accumulate), followed by per-channel
  * thresholds: code = #{k : acc >= thresholds[c][k]}.

@@ -6,6 +6,7 @@
 #include "apnn_oracle.h"
 
 #include <stdlib.h>
+#include <math.h>
 #include <string.h>
 
 /* ---------------------------------------------------------------------------------------- */
@@ -265,6 +266,22 @@ void oracle_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C,
         const uint32_t bit = (values[(size_t)r * C + c] >> b) & 1u;
         planes[(size_t)b * rows * cw + (size_t)r * cw + c / 32] |= bit << (31 - (c % 32));
       }
+}
+
+void oracle_quantize_val(const float *x, uint32_t *q, long long n, int bits, float min_v, float max_v) {
+  const uint32_t top = (1u << bits) - 1u;
+  const float levels = (float)(1 << bits), range = max_v - min_v;
+  for (long long i = 0; i < n; i++) {
+    float v = x[i];
+    v = v < min_v ? min_v : (v > max_v ? max_v : v);
+    volatile float a = v - min_v;   /* volatile: one rounding per operation, as on the device */
+    volatile float b = a * levels;
+    volatile float c = b * 1.0f;
+    volatile float d = c / range;
+    const float r = rintf(d);       /* default rounding mode: to nearest, ties to even */
+    const uint32_t code = (uint32_t)r;
+    q[i] = code > top ? top : code;
+  }
 }
 
 void oracle_unpack_bits(const uint32_t *planes, uint32_t *values, int rows, int C, int cpad, int bits) {

@@ -112,6 +112,12 @@ void oracle_bn_quantize(const int32_t *acc, const int32_t *resid, const int32_t 
  * per element) -> planes [bits][rows][cpad/32], channel c at bit 31 - c%32, pad channels zero. */
 void oracle_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits);
 
+/* Affine quantizer of NN/kernel.cuh:29-44 (Quantize_val), fp32, same operation order, round half to
+ * even, clamped to the top code: q = min(2^bits-1, rint(((clip(x)-min_v) * 2^bits * 1.0f) / (max_v-min_v))).
+ * Pinned by closed forms (end points, exact mid-levels, monotonicity) and by an independent numpy
+ * float32 evaluation in tests/test_oracle.py; the reference never stores this value (kernel.cuh:42). */
+void oracle_quantize_val(const float *x, uint32_t *q, long long n, int bits, float min_v, float max_v);
+
 /* Inverse of oracle_pack_bits (NN/param.h:634-658 shows the (r>>(31-lane))&1 indexing). */
 void oracle_unpack_bits(const uint32_t *planes, uint32_t *values, int rows, int C, int cpad, int bits);
 

@@ -52,13 +52,15 @@ def lib():
         L.oracle_maxpool2x2.argtypes = [i32p, i32p, ci, ci, ci, ci]
         L.oracle_bn_quantize.argtypes = [i32p, i32p, i32p, u8p, i32p, ci, ci, ci]
         L.oracle_pack_bits.argtypes = [u32p, u32p, ci, ci, ci, ci]
+        L.oracle_quantize_val.argtypes = [ctypes.POINTER(ctypes.c_float), u32p, ctypes.c_longlong, ci, ctypes.c_float,
+                                          ctypes.c_float]
         L.oracle_unpack_bits.argtypes = [u32p, u32p, ci, ci, ci, ci]
         L.oracle_conv_i8.argtypes = [i8p, i8p, i32p] + [ci] * 9
         L.oracle_fnv1a64.argtypes = [ctypes.c_void_p, ctypes.c_uint64]
         L.oracle_fnv1a64.restype = ctypes.c_uint64
         for f in ("oracle_gemm_literal", "oracle_gemm", "oracle_gemm_rows", "oracle_conv3x3_literal",
                   "oracle_conv", "oracle_lowbits_pack", "oracle_avgpool2x2", "oracle_maxpool2x2",
-                  "oracle_bn_quantize", "oracle_pack_bits", "oracle_unpack_bits", "oracle_conv_i8"):
+                  "oracle_bn_quantize", "oracle_pack_bits", "oracle_unpack_bits", "oracle_conv_i8", "oracle_quantize_val"):
             getattr(L, f).restype = None
         _lib = L
     return _lib
@@ -145,6 +147,13 @@ def pack_bits(values, rows, C, cpad, bits):
     planes = np.empty((bits, rows, cpad // 32), np.uint32)
     lib().oracle_pack_bits(_p(values, u32p), _p(planes, u32p), rows, C, cpad, bits)
     return planes
+
+
+def quantize_val(x, bits, min_v=-10.0, max_v=10.0):
+    x = np.ascontiguousarray(x, np.float32)
+    q = np.empty(x.shape, np.uint32)
+    lib().oracle_quantize_val(x.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), _p(q, u32p), x.size, bits, min_v, max_v)
+    return q
 
 
 def unpack_bits(planes, rows, C, cpad, bits):

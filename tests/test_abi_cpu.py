@@ -108,3 +108,42 @@ def test_combinations_that_are_not_built_are_reported():
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL                # at most 8 planes per operand
     g.wb, g.xb, g.path = 1, 2, A.PATH_VALU | (9 << 8)
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL                # no such tile
+
+
+def test_fold_bn_matches_double_precision_brute_force():
+    """apnn_fold_bn is host-only: thresholds + flip reproduce clamp(floor(y / step)) of the double-precision
+    batch-norm for every accumulator value in a range (rising, falling and constant channels)."""
+    import numpy as np
+    import oracle_lib as O
+    L = A.lib()
+    rng = np.random.default_rng(77)
+    C = 24
+    for bits, step, in_scale in [(1, 0.5, 1.0), (2, 0.7, 0.25), (3, 0.31, 2.0), (4, 0.2, -1.0)]:
+        gamma = (rng.uniform(0.3, 2.0, C) * rng.choice([-1.0, 1.0], C)).astype(np.float32)
+        gamma[3] = 0.0
+        beta = rng.uniform(-1, 1, C).astype(np.float32)
+        mean = rng.uniform(-20, 20, C).astype(np.float32)
+        var = rng.uniform(4, 900, C).astype(np.float32)
+        eps = np.float32(1e-5)
+        nt = 2 ** bits - 1
+        thr = np.zeros((C, nt), np.int32)
+        flip = np.zeros(C, np.uint8)
+        p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+        rc = L.apnn_fold_bn(p(gamma), p(beta), p(mean), p(var), eps, in_scale, step, C, bits, p(thr), p(flip))
+        assert rc == 0
+        assert np.all(np.diff(thr.astype(np.int64), axis=1) >= 0)
+        v = np.arange(-700, 700, dtype=np.int32)
+        acc = np.repeat(v[:, None], C, axis=1)
+        slope = gamma.astype(np.float64) / np.sqrt(var.astype(np.float64) + np.float64(eps))
+        y = slope[None, :] * (acc.astype(np.float64) * np.float64(np.float32(in_scale)) - mean.astype(np.float64)[None, :]) \
+            + beta.astype(np.float64)[None, :]
+        expect = np.clip(np.floor(y / np.float64(np.float32(step))), 0, nt).astype(np.int32)
+        # y >= k*step  <=>  floor(y/step) >= k  holds in exact arithmetic; skip values within rounding of a level
+        q = O.bn_quantize(acc, None, thr, flip, bits)
+        frac = y / np.float64(np.float32(step))
+        safe = np.abs(frac - np.rint(frac)) > 1e-9
+        assert np.array_equal(q[safe], expect[safe])
+        assert flip[3] == 0 and set(np.unique(q[:, 3])) <= {int(expect[0, 3])}
+    bad = np.zeros(4, np.float32)
+    assert L.apnn_fold_bn(None, p(bad), p(bad), p(bad), eps, 1.0, 1.0, 4, 2, p(thr), p(flip)) == A.ENULL
+    assert L.apnn_fold_bn(p(bad), p(bad), p(bad), p(bad), eps, 1.0, 0.0, 4, 2, p(thr), p(flip)) == A.EINVAL

@@ -604,3 +604,19 @@ def test_any_precision_descriptor_paths(G, wb, xb, ob, sym):
     assert np.array_equal(G.run_conv(Wc, Xc, cin_pad=C, sym=sym, **kw).reshape(expect.shape), expect)
     with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):
         G.run_conv(Wc, Xc, cin_pad=C, sym=sym, path=4, **kw)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("rows,C,cpad", [(37, 3, 32), (50, 70, 128), (8, 256, 256)])
+def test_quantize_pack(G, bits, rows, C, cpad):
+    """Float image / feature map -> affine codes -> bit-planes in one kernel (Quantize_val + Bit_compression)."""
+    rng = np.random.default_rng(6000 + bits + rows)
+    x = rng.uniform(-12, 12, size=(rows, C)).astype(np.float32)
+    x[0, :] = np.linspace(-10, 10, C, dtype=np.float32)            # includes both end points
+    x[1, :] = (-10.0 + 20.0 * (np.arange(C) % (2 ** bits) + 0.5) / 2 ** bits).astype(np.float32)   # ties
+    dX = torch.from_numpy(x).cuda()
+    planes = G.dev_empty_i32(bits * rows * cpad // 32, fill=-7)
+    G.A.check(G.A.lib().apnn_quantize_pack(G.ptr(dX), G.ptr(planes), rows, C, cpad, bits, -10.0, 10.0, None), "quantize_pack")
+    codes = O.quantize_val(x, bits)
+    expect = O.pack_bits(codes, rows, C, cpad, bits)
+    assert np.array_equal(G.to_host(planes, np.uint32).reshape(expect.shape), expect)

@@ -236,3 +236,33 @@ def test_conv_i8_vs_numpy():
     got = O.conv_i8(Wt, X, 2, 3)
     expect = _np_conv(X.astype(np.int64), Wt.astype(np.int64), 2, 3)
     assert np.array_equal(got, expect)
+
+
+def test_quantize_val_closed_forms_and_numpy_float32():
+    """Quantize_val (NN/kernel.cuh:29-44): end points, exact levels, ties, monotonicity, and an independent
+    float32 evaluation of the same expression."""
+    for bits in (1, 2, 4, 8):
+        top = 2 ** bits - 1
+        x = np.array([-1e9, -10.0, 10.0, 1e9, 0.0], np.float32)
+        q = O.quantize_val(x, bits)
+        assert list(q) == [0, 0, top, top, min(top, 2 ** (bits - 1))]     # clip, clamp, mid level
+        # x = -10 + 20*k/2^bits is exactly level k; half way between two levels rounds to the even one
+        k = np.arange(0, 2 ** bits + 1)
+        xs = (-10.0 + 20.0 * k / 2 ** bits).astype(np.float32)
+        assert np.array_equal(O.quantize_val(xs, bits), np.minimum(k, top))
+        if bits <= 4:
+            ties = (-10.0 + 20.0 * (k[:-1] + 0.5) / 2 ** bits).astype(np.float32)   # exactly representable
+            expect = np.minimum(np.where(k[:-1] % 2 == 0, k[:-1], k[:-1] + 1), top)
+            assert np.array_equal(O.quantize_val(ties, bits), expect)
+        rng = np.random.default_rng(40 + bits)
+        r = np.sort(rng.uniform(-12, 12, 5000).astype(np.float32))
+        qr = O.quantize_val(r, bits)
+        assert np.all(np.diff(qr.astype(np.int64)) >= 0)
+        f = np.float32
+        c = np.clip(r, f(-10), f(10))
+        ref = np.rint(((c - f(-10)) * f(2 ** bits) * f(1.0)) / f(20.0))
+        assert np.array_equal(qr, np.minimum(ref, top).astype(np.uint32))
+    # other ranges
+    x = np.linspace(-1, 3, 1001).astype(np.float32)
+    q = O.quantize_val(x, 3, 0.0, 2.0)
+    assert q[0] == 0 and q[-1] == 7 and np.all(np.diff(q.astype(np.int64)) >= 0)
