@@ -29,6 +29,9 @@
  *   bn_quantize                    a=1 special case == (acc >= t) of NN/kernel.cuh:833-834;
  *                                  multi-bit form is defined by this build                 : parity unpinned beyond a=1
  *   pack_bits                      round trip + hand-written words (NN/kernel.cuh:58-76)   : pinned
+ *   quantize_val                   end points, exact levels, ties-to-even, monotonicity and an
+ *                                  independent numpy float32 evaluation (NN/kernel.cuh:29-44; the
+ *                                  reference never stores its result, so no reference output exists) : pinned by arithmetic only
  */
 #ifndef APNN_ORACLE_H
 #define APNN_ORACLE_H
