@@ -419,10 +419,11 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
     rd[j] = idx < npatch ? ((r << 16) | (idx - r * NDW)) : -1;
   }
   uint32_t raw[NSLOT];
-  auto request = [&](long long grp, int base) {
-    const int gx = (int)(grp % gpr);
-    const int oy = (int)((grp / gpr) % Ho);
-    const int b = (int)(grp / ((long long)gpr * Ho));
+  auto request = [&](uint32_t grp, int base) {
+    const uint32_t trow = grp / (uint32_t)gpr;
+    const int gx = (int)(grp - trow * (uint32_t)gpr);
+    const int b = (int)(trow / (uint32_t)Ho);
+    const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
     const int sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
     const uint8_t *img = X + (long long)b * H * rowbytes;
 #pragma unroll
@@ -458,19 +459,21 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
     }
   };
 
-  const long long gstep = (long long)gridDim.x * 4;
-  long long group = (long long)blockIdx.x * 4 + wave;
-  if (prefetch && group < ngroups) request(group, 0);
-  for (; group < ngroups; group += gstep) {
-    const int gx = (int)(group % gpr);
-    const int oy = (int)((group / gpr) % Ho);
-    const int b = (int)(group / ((long long)gpr * Ho));
+  // (the launcher keeps the number of groups below 2^31: 32-bit index arithmetic)
+  const uint32_t gstep = gridDim.x * 4u, ng = (uint32_t)ngroups;
+  uint32_t group = blockIdx.x * 4u + (uint32_t)wave;
+  if (prefetch && group < ng) request(group, 0);
+  for (; group < ng; group += gstep) {
+    const uint32_t trow = group / (uint32_t)gpr;
+    const int gx = (int)(group - trow * (uint32_t)gpr);
+    const int b = (int)(trow / (uint32_t)Ho);
+    const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
     const int ox0 = gx * 32;
     const int s0 = (ox0 * stride - pad) * C;
     const int lead = s0 - (s0 & ~3);
     if (prefetch) {
       publish(0);
-      if (group + gstep < ngroups) request(group + gstep, 0);
+      if (group + gstep < ng) request(group + gstep, 0);
     } else {
       for (int base = 0; base < npatch; base += 64 * NSLOT) {
         request(group, base);
@@ -565,11 +568,26 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__rest
                                                           int pad, int Ho, int Wo) {
   const long long rows_in = (long long)B * H * W, rows_out = (long long)B * Ho * Wo;
   const long long total = rows_out * cw;
+  const bool small = total < 0x7fffffffLL;  // 32-bit index arithmetic (64-bit divisions cost ~100 instructions)
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (long long)gridDim.x * blockDim.x) {
-    const int wi = (int)(i % cw);
-    const long long row = i / cw;
-    const int ox = (int)(row % Wo), oy = (int)((row / Wo) % Ho), b = (int)(row / ((long long)Wo * Ho));
+    int wi, ox, oy, b;
+    long long row;
+    if (small) {
+      const uint32_t iu = (uint32_t)i, r32 = iu / (uint32_t)cw;
+      wi = (int)(iu - r32 * (uint32_t)cw);
+      const uint32_t t = r32 / (uint32_t)Wo;
+      ox = (int)(r32 - t * (uint32_t)Wo);
+      b = (int)(t / (uint32_t)Ho);
+      oy = (int)(t - (uint32_t)b * (uint32_t)Ho);
+      row = r32;
+    } else {
+      wi = (int)(i % cw);
+      row = i / cw;
+      ox = (int)(row % Wo);
+      oy = (int)((row / Wo) % Ho);
+      b = (int)(row / ((long long)Wo * Ho));
+    }
     uint32_t m[8];
 #pragma unroll
     for (int p = 0; p < 8; ++p) m[p] = 0;
@@ -650,8 +668,16 @@ __global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restr
   // every lane of a JP-group runs the same number of iterations (the shuffles need all of them)
   for (long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x; t / JP < total; t += nthreads) {
     const long long i = t / JP;
-    const long long r = i / C;
-    const int c = (int)(i % C);
+    long long r;
+    int c;
+    if (total < 0x7fffffffLL) {
+      const uint32_t r32 = (uint32_t)i / (uint32_t)C;
+      c = (int)((uint32_t)i - r32 * (uint32_t)C);
+      r = r32;
+    } else {
+      r = i / C;
+      c = (int)(i % C);
+    }
     const int sh = 31 - (c & 31);
     int sum = 0;
     for (int j = part; j < group; j += JP) {
@@ -724,6 +750,7 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
   const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
   dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
   if (C <= 4 && planes != nullptr && codes == nullptr && acc_out == nullptr && bits <= 2 && (COUT % 32) == 0 &&
+      groups < 0x7fffffffLL &&
       ((W * C) % 4) == 0 && (reinterpret_cast<uintptr_t>(X) & 3u) == 0 && (zero_point == 0 || zero_point == 128) &&
       thr != nullptr) {
     // image rows consumed as bytes (no repacking): see conv_i8_rows_kernel
