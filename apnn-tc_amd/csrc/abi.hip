@@ -213,6 +213,9 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
     const int big = conv ? 7 : 6;
     if (ntiles(big) >= cus && fill(big) >= 0.8) return big;
     if (ntiles(1) >= cus && fill(1) >= 0.8) return 1;
+    // convolution: 128 pixels x 64 channels per work-group (one activation expansion feeds two
+    // blocks per wave) measures faster than 64x64 whenever it still fills the chip
+    if (conv && ntiles(3) >= cus && fill(3) >= 0.8) return 3;
   }
   if (ntiles(2) >= cus / 2 || KW < 16) return 2;
   return ntiles(5) >= cus / 2 ? 5 : 4;
