@@ -295,6 +295,13 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
+  const bool direct_ok = d->epi.mode == APNN_EPI_INT32 && fn != apnn::valu_gemm_any_x && (p.rowsB & 3) == 0 &&
+                         p.KW <= 64;
+  if (tile_pin == apnn::TILE_DIRECT + 1)  // register-only kernel: int32 output, K <= 2048
+    return direct_ok ? from_hip(fn(4, apnn::TILE_DIRECT, p, stream)) : APNN_EUNSUPPORTED;
+  // small, latency-bound problems (the M = 64 sweep): one round of loads, no LDS, no barrier
+  if (tile_pin == 0 && direct_ok && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
+    return from_hip(fn(4, apnn::TILE_DIRECT, p, stream));
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
   return (int)fn(4, tile, p, stream);
 }

@@ -9,7 +9,8 @@
 
 namespace apnn {
 
-enum TileSel { TILE_64x64 = 0, TILE_32x32 = 1, TILE_16x32 = 2, TILE_16x16 = 3, TILE_COUNT = 4 };
+// TILE_DIRECT: the register-only kernel of valu_direct_kernel.h (GEMM entry points, int32 output)
+enum TileSel { TILE_64x64 = 0, TILE_32x32 = 1, TILE_16x32 = 2, TILE_16x16 = 3, TILE_COUNT = 4, TILE_DIRECT = 4 };
 
 struct KParams {
   const uint32_t *A;

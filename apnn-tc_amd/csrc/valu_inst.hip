@@ -1,5 +1,6 @@
 // One translation unit per (INST_PA, INST_PB, INST_CONV), selected on the compiler command line,
 // so that the tile-shape instantiations of the VALU kernel build in parallel.
+#include "valu_direct_kernel.h"
 #include "valu_kernel.h"
 
 #ifndef INST_PA
@@ -22,6 +23,7 @@ hipError_t APNN_CAT(valu_conv_, INST_PA, INST_PB, x)(int vw, int tile, const KPa
 #else
 hipError_t APNN_CAT(valu_gemm_, INST_PA, INST_PB, x)(int vw, int tile, const KParams &p, hipStream_t s) {
   (void)vw;  // GEMM rows are whole int4 words (K % 128 == 0)
+  if (tile == TILE_DIRECT) return launch_valu_direct<INST_PA, INST_PB>(p, s);
   return launch_valu_tile<INST_PA, INST_PB, 4, false>(tile, p, s);
 }
 #endif

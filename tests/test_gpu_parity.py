@@ -620,3 +620,28 @@ def test_quantize_pack(G, bits, rows, C, cpad):
     codes = O.quantize_val(x, bits)
     expect = O.pack_bits(codes, rows, C, cpad, bits)
     assert np.array_equal(G.to_host(planes, np.uint32).reshape(expect.shape), expect)
+
+
+@pytest.mark.parametrize("sym", [0, 1])
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (50, 36, 128), (1, 4, 2048), (64, 128, 1536), (7, 260, 640)])
+def test_gemm_register_only_kernel(G, M, N, K, wb, xb, sym):
+    """The latency-oriented GEMM kernel (eight lanes split K for four outputs), pinned as VALU tile 4."""
+    rng = np.random.default_rng(7000 + M + N + K + 10 * wb + xb + sym)
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=1, tile=4).reshape(M, N)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=sym))
+
+
+def test_gemm_register_only_kernel_limits(G):
+    rng = np.random.default_rng(7100)
+    W = O.random_planes(rng, 1, 8, 4096 // 32)
+    X = O.random_planes(rng, 2, 8, 4096 // 32)
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):     # K > 2048
+        G.run_gemm(W, X, 8, 8, 4096, 1, 2, path=1, tile=4)
+    W = O.random_planes(rng, 1, 8, 4)
+    X = O.random_planes(rng, 2, 6, 4)
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):     # N % 4 != 0
+        G.run_gemm(W, X, 8, 6, 128, 1, 2, path=1, tile=4)
+    assert np.array_equal(G.run_gemm(W, X, 8, 6, 128, 1, 2).reshape(8, 6), O.gemm(W, X, 8, 6, 128, 1, 2))
