@@ -490,7 +490,10 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   using FragT = typename std::conditional<F4, v8i, v4i>::type;
   constexpr int NT = 256;
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr int KC = 8;              // k-words (32 elements each) per staged chunk
+  // k-words (32 elements each) per staged chunk.  The convolution kernels whose waves tile the output
+  // (64x64 and 128x64 per work-group; larger tiles measure no gain) stage 16: their per-chunk work (im2col addressing, LDS staging, barrier) is a large share of a
+  // short K loop, and k-steps past the end of K are skipped, so a longer chunk wastes nothing.
+  constexpr int KC = (CONV && KS == 1 && FA * FB <= 2) ? 16 : 8;
   constexpr int LD = KC + 1;         // odd row pitch: 32 rows hit 32 different banks
   constexpr int KQ = KC / VW;
   constexpr int UA = TA * KQ, UB = TB * KQ;
@@ -754,9 +757,11 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
         __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);  // then its share of VALU work
       }
     };
-    // k-steps 0 .. NKS-2 (kept as a real loop: one scheduling region per k-step)
+    // k-steps of this chunk that hold data (the last chunk may be short)
+    const int nks = min(NKS, (p.KW - ch * KC + WPS - 1) / WPS);
+    // k-steps 0 .. nks-2 (kept as a real loop: one scheduling region per k-step)
 #pragma unroll 1
-    for (int ks = 0; ks + 1 < NKS; ++ks) {
+    for (int ks = 0; ks + 1 < nks; ++ks) {
       read_words(cur, ks + 1);
       mfma_all();
       advance();
@@ -780,8 +785,9 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
 }
 
-constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB) {
-  const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * 9 * sizeof(uint32_t);
+constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB, bool conv) {
+  const size_t ld = (conv && WA * WB == 4 && FA * FB <= 2) ? 17 : 9;  // KC + 1, see the kernel
+  const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
   const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
   return stage > slab ? stage : slab;
 }
@@ -790,7 +796,7 @@ constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB)
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr size_t smem_bytes = mfma_smem_bytes(PA, PB, FA, FB, WA, WB);
+  constexpr size_t smem_bytes = mfma_smem_bytes(PA, PB, FA, FB, WA, WB, CONV);
   constexpr int OCC = (OCC_WANTED > 1 && smem_bytes * OCC_WANTED <= 160 * 1024) ? OCC_WANTED : 1;
   static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
   auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>;
