@@ -762,7 +762,11 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
     const size_t lds = (size_t)64 * (nks * 32 + 16) + 4 * (size_t)R * PWD * 4;
     if (lds <= 64 * 1024) {
       // persistent grid: exactly as many work-groups as the device holds at once
-      auto kern = nks == 7 ? conv_i8_rows_kernel<7> : conv_i8_rows_kernel<0>;
+      // Filter block in registers (two work-groups per compute unit fit) while one or two rounds of
+      // work-groups cover all pixel groups; beyond that the variant that re-reads the filter from LDS
+      // wins through its higher occupancy (four per compute unit).
+      const bool wreg = nks == 7 && grid.x <= 1024;
+      auto kern = wreg ? conv_i8_rows_kernel<7> : conv_i8_rows_kernel<0>;
       int per_cu = 0, cus = 0, dev = 0;
       hipError_t e = hipGetDevice(&dev);
       if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -775,7 +779,7 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
       dim3 g2(grid.x > resident ? resident : grid.x, grid.y);
       const uint32_t xm = zero_point == 128 ? 0x80808080u : 0u;
       const uint8_t *Xu = reinterpret_cast<const uint8_t *>(X);
-      if (nks == 7)
+      if (wreg)
         hipLaunchKernelGGL(conv_i8_rows_kernel<7>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
                            stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD);
       else
