@@ -39,9 +39,84 @@ int timed_loop(F &&launch, int warmup, int iters, hipStream_t stream, float *eve
   return rc;
 }
 
+// Same measurement with the launches replayed from a HIP graph: `batch` launches are captured once
+// (on a stream of its own, default priority) and the graph is launched ceil(n / batch) times, the last
+// time through a second graph holding the remainder, so exactly `warmup` + `iters` kernels run.  The
+// host then issues one graph launch per `batch` kernels instead of one call per kernel.
+template <class F>
+int timed_graph_loop(F &&launch_on, int warmup, int iters, int batch, float *event_ms, double *wall_ms) {
+  if (batch < 1) batch = 1;
+  hipStream_t cs = nullptr;
+  hipError_t err = hipStreamCreateWithFlags(&cs, hipStreamNonBlocking);
+  if (err != hipSuccess) return (int)err;
+  hipGraphExec_t full = nullptr, rest_w = nullptr, rest_i = nullptr;
+  int rc = 0;
+  auto capture = [&](int n, hipGraphExec_t *exec) -> int {
+    if (n <= 0) return 0;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamBeginCapture(cs, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return (int)e;
+    int r = 0;
+    for (int i = 0; i < n && r == 0; ++i) r = launch_on(cs);
+    e = hipStreamEndCapture(cs, &g);
+    if (r != 0) return r;
+    if (e != hipSuccess) return (int)e;
+    e = hipGraphInstantiate(exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    return (int)e;
+  };
+  const int nfull_needed = (warmup >= batch || iters >= batch) ? batch : 0;
+  if ((rc = capture(nfull_needed, &full)) == 0 && (rc = capture(warmup % batch, &rest_w)) == 0)
+    rc = capture(iters % batch, &rest_i);
+  auto replay = [&](int n, hipGraphExec_t rest) -> int {
+    for (int i = 0; i < n / batch; ++i) {
+      const hipError_t e = hipGraphLaunch(full, cs);
+      if (e != hipSuccess) return (int)e;
+    }
+    if (n % batch) {
+      const hipError_t e = hipGraphLaunch(rest, cs);
+      if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+  };
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (rc == 0 && (err = hipEventCreate(&e0)) != hipSuccess) rc = (int)err;
+  if (rc == 0 && (err = hipEventCreate(&e1)) != hipSuccess) rc = (int)err;
+  if (rc == 0) rc = replay(warmup, rest_w);
+  if (rc == 0 && (err = hipStreamSynchronize(cs)) != hipSuccess) rc = (int)err;
+  if (rc == 0) {
+    const auto t0 = std::chrono::steady_clock::now();
+    (void)hipEventRecord(e0, cs);
+    rc = replay(iters, rest_i);
+    (void)hipEventRecord(e1, cs);
+    err = hipStreamSynchronize(cs);
+    const auto t1 = std::chrono::steady_clock::now();
+    if (rc == 0 && err != hipSuccess) rc = (int)err;
+    if (rc == 0) {
+      float ms = 0.f;
+      (void)hipEventElapsedTime(&ms, e0, e1);
+      *event_ms = ms;
+      *wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (full) (void)hipGraphExecDestroy(full);
+  if (rest_w) (void)hipGraphExecDestroy(rest_w);
+  if (rest_i) (void)hipGraphExecDestroy(rest_i);
+  (void)hipStreamDestroy(cs);
+  return rc;
+}
+
 }  // namespace
 
 extern "C" {
+
+// apnn_bench_gemm with the launches replayed from HIP graphs of `batch` launches each.
+int apnn_bench_gemm_graph(const apnn_gemm_desc *d, int warmup, int iters, int batch, float *event_ms,
+                          double *wall_ms) {
+  return timed_graph_loop([&](hipStream_t cs) { return apnn_gemm(d, cs); }, warmup, iters, batch, event_ms, wall_ms);
+}
 
 // Runs `iters` back-to-back apnn_gemm launches of the same descriptor on `stream` after `warmup`
 // untimed ones.  event_ms: HIP-event time over the timed launches; wall_ms: host wall clock from
@@ -50,6 +125,11 @@ int apnn_bench_gemm(const apnn_gemm_desc *d, int warmup, int iters, apnn_stream_
                     double *wall_ms) {
   hipStream_t stream = static_cast<hipStream_t>(s);
   return timed_loop([&]() { return apnn_gemm(d, s); }, warmup, iters, stream, event_ms, wall_ms);
+}
+
+int apnn_bench_conv_graph(const apnn_conv_desc *d, int warmup, int iters, int batch, float *event_ms,
+                          double *wall_ms) {
+  return timed_graph_loop([&](hipStream_t cs) { return apnn_conv(d, cs); }, warmup, iters, batch, event_ms, wall_ms);
 }
 
 int apnn_bench_conv(const apnn_conv_desc *d, int warmup, int iters, apnn_stream_t s, float *event_ms,

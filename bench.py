@@ -5,7 +5,11 @@ Headline metric (BASELINE.json): w1a2 GEMM effective TOPS at M=64, N=K=1024, wei
 as one bit (w = 2b-1), activations unsigned 2-bit, bit-packed along K, int32 output.  One "step" is
 one launch of that GEMM through the C ABI with all operands resident in HBM.  The timed loop runs in
 C++ (libapnn_bench.so), like the timing section of the reference's benchmark main
-(APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:526-549).
+(APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:526-549).  The launches of the
+latency-bound shapes (headline, M=64 sweep, batch-1 convolutions) are replayed from HIP graphs of
+GRAPH_BATCH launches each: a plain host loop of thousands of ~3 us launches is throttled by the host
+side of the queue (3.0-4.4 us per launch depending on the loop length), graph replay issues the same
+kernels at the device's own rate.  The plain-loop figure is reported beside it.
 
 Prints ONE JSON line.  Besides the contract fields it carries
   roofline     : the GEMM kernel against the HBM roofline (algorithmic bytes / HIP-event time per launch)
@@ -30,6 +34,7 @@ FP4_MFMA_PEAK_TOPS = 10100.0   # MI355X dense fp4 MFMA (the matrix-core path fee
 # calibration, WRITE_SIZE 256 KiB x 1.0): see profiles/gemm_w1a2_m64_n1024_k1024.md
 HEADLINE_TRAFFIC_BYTES = 652357
 BASELINE_TOPS = 18.66          # reference README.md:142 (w1a2, M=64, N=K=1024, sm_86)
+GRAPH_BATCH = 200              # kernel launches per captured HIP graph
 
 
 def gemm_bytes(M, N, K, wb, xb):
@@ -72,6 +77,10 @@ def main():
                                          ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     benchlib.apnn_bench_conv.argtypes = [ctypes.POINTER(A.ConvDesc), ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                          ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    benchlib.apnn_bench_gemm_graph.argtypes = [ctypes.POINTER(A.GemmDesc), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    benchlib.apnn_bench_conv_graph.argtypes = [ctypes.POINTER(A.ConvDesc), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     benchlib.apnn_bench_empty.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                           ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -83,7 +92,7 @@ def main():
         X = O.random_planes(np.random.default_rng(0x5EED0002), xb, N, K // 32)
         return W, X
 
-    def time_gemm(M, N, K, wb, xb, sym, warmup, iters, verify_rows=None):
+    def time_gemm(M, N, K, wb, xb, sym, warmup, iters, verify_rows=None, graph=False):
         W, X = make_inputs(M, N, K, wb, xb)
         dW, dX = G.to_dev(W), G.to_dev(X)
         out = G.dev_empty_i32(M * N, fill=-7)
@@ -91,8 +100,12 @@ def main():
                        weight_mode=sym, path=path)
         ev, wall = ctypes.c_float(), ctypes.c_double()
         torch.cuda.synchronize()
-        A.check(benchlib.apnn_bench_gemm(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
-                                         ctypes.byref(wall)), "apnn_bench_gemm")
+        if graph:
+            A.check(benchlib.apnn_bench_gemm_graph(ctypes.byref(d), warmup, iters, GRAPH_BATCH, ctypes.byref(ev),
+                                                   ctypes.byref(wall)), "apnn_bench_gemm_graph")
+        else:
+            A.check(benchlib.apnn_bench_gemm(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
+                                             ctypes.byref(wall)), "apnn_bench_gemm")
         torch.cuda.synchronize()
         got = G.to_host(out).reshape(M, N)
         if verify_rows is None:
@@ -116,7 +129,7 @@ def main():
     M, N, K, wb, xb = 64, 1024, 1024, 1, 2
     ops = 2.0 * M * N * K
     nbytes = gemm_bytes(M, N, K, wb, xb)
-    r = time_gemm(M, N, K, wb, xb, A.WEIGHT_SYMMETRIC, args.warmup, args.steps)
+    r = time_gemm(M, N, K, wb, xb, A.WEIGHT_SYMMETRIC, args.warmup, args.steps, graph=True)
     tops = ops / (r["wall_ms"] * 1e-3) / 1e12
     achieved_gbs = nbytes / (r["event_ms"] * 1e-3) / 1e9
     result = {
@@ -133,19 +146,25 @@ def main():
         "dtype": "int32 accumulate over 1-bit x 2-bit planes",
         "data": "synthetic",
         "config": {"workload": "apnn_gemm w1a2 M=64 N=1024 K=1024, weights 2b-1 (symmetric), int32 out",
-                   "path": args.path, "verified_bit_exact": r["verified"]},
+                   "path": args.path, "launch": "HIP graph replay, %d launches per graph" % GRAPH_BATCH,
+                   "verified_bit_exact": r["verified"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 3), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 6), "traffic": HEADLINE_TRAFFIC_BYTES,
                      "algorithmic_bytes": nbytes, "kernel_us": round(r["event_ms"] * 1e3, 4)},
     }
 
     extra = {}
+    # the reference's unsigned arithmetic right after the headline run (same clock state: a loop of
+    # empty kernels in between lets the GPU clock down and the next short measurement pays for it)
+    ru = time_gemm(M, N, K, wb, xb, A.WEIGHT_UNSIGNED, args.warmup, args.steps, graph=True)
+    extra["unsigned_reference_arithmetic"] = {"tops": round(ops / (ru["wall_ms"] * 1e-3) / 1e12, 4),
+                                              "us": round(ru["wall_ms"] * 1e3, 4), "verified": ru["verified"]}
+    re_ = time_gemm(M, N, K, wb, xb, A.WEIGHT_SYMMETRIC, args.warmup, args.steps)
+    extra["plain_launch_loop"] = {"tops": round(ops / (re_["wall_ms"] * 1e-3) / 1e12, 4),
+                                  "us": round(re_["wall_ms"] * 1e3, 4), "verified": re_["verified"]}
     ev, wall = ctypes.c_float(), ctypes.c_double()
     benchlib.apnn_bench_empty(args.warmup, args.steps, stream, ctypes.byref(ev), ctypes.byref(wall))
     extra["empty_kernel_us_per_launch"] = round(wall.value / args.steps * 1e3, 4)
-    ru = time_gemm(M, N, K, wb, xb, A.WEIGHT_UNSIGNED, args.warmup, args.steps)
-    extra["unsigned_reference_arithmetic"] = {"tops": round(ops / (ru["wall_ms"] * 1e-3) / 1e12, 4),
-                                              "us": round(ru["wall_ms"] * 1e3, 4), "verified": ru["verified"]}
 
     def time_conv(batch, C, w_, a_, fused, warmup, iters):
         """3x3, stride 1, stored halo, 16x16 feature map, Cin = Cout = C (the reference's conv benchmark,
@@ -173,8 +192,12 @@ def main():
                        R=3, S=3, stride=1, pad=1, halo=1, wb=w_, xb=a_, weight_mode=A.WEIGHT_UNSIGNED, epi=E,
                        path=path)
         ev, wall = ctypes.c_float(), ctypes.c_double()
-        A.check(benchlib.apnn_bench_conv(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
-                                         ctypes.byref(wall)), "apnn_bench_conv")
+        if batch == 1:
+            A.check(benchlib.apnn_bench_conv_graph(ctypes.byref(d), warmup, iters, GRAPH_BATCH, ctypes.byref(ev),
+                                                   ctypes.byref(wall)), "apnn_bench_conv_graph")
+        else:
+            A.check(benchlib.apnn_bench_conv(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
+                                             ctypes.byref(wall)), "apnn_bench_conv")
         torch.cuda.synchronize()
         ok = None
         if not fused and batch * C <= 1024:
@@ -190,7 +213,7 @@ def main():
         shapes = []
         for (w_, a_) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
             for nk in (128, 256, 384, 512, 640, 768, 896, 1024) if on("gemm_sweep") else ():
-                t = time_gemm(64, nk, nk, w_, a_, A.WEIGHT_UNSIGNED, 20, 200)
+                t = time_gemm(64, nk, nk, w_, a_, A.WEIGHT_UNSIGNED, 200, 2000, graph=True)
                 shapes.append({"shape": "w%da%d M=64 N=K=%d" % (w_, a_, nk),
                                "us": round(t["wall_ms"] * 1e3, 3),
                                "tops": round(2.0 * 64 * nk * nk / (t["wall_ms"] * 1e-3) / 1e12, 3),
