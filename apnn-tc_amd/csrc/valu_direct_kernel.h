@@ -26,11 +26,13 @@ template <int PA, int PB, int NQ>
 __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) {
   const int tid = threadIdx.x;
   const int l = tid & 7;                               // K slice
-  const long long grp = ((long long)blockIdx.x * 256 + tid) >> 3;
-  const int groups_per_row = p.rowsB >> 2;
-  const int a = (int)(grp / groups_per_row);
-  const int b = (int)(grp - (long long)a * groups_per_row) << 2;
-  const bool live = a < p.rowsA;
+  // a work-group covers four output rows x 32 columns (one row per wave): its waves read the same 32
+  // rows of B, so three of the four reads hit the compute unit's L1
+  const int chunks_b = (p.rowsB + 31) >> 5;
+  const int ab = blockIdx.x / chunks_b, bc = blockIdx.x - ab * chunks_b;
+  const int a = ab * 4 + (tid >> 6);
+  const int b = bc * 32 + ((tid & 63) >> 3) * 4;
+  const bool live = a < p.rowsA && b < p.rowsB;
   const int nq = p.KW >> 2;                            // 128-bit groups per row
 
   uint4 wa[PA][NQ], xb[4][PB][NQ];
@@ -85,8 +87,7 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
 template <int PA, int PB>
 inline hipError_t launch_valu_direct(const KParams &p, hipStream_t stream) {
   if ((p.rowsB & 3) != 0 || (p.KW & 3) != 0 || p.KW > 32 * DIRECT_MAXQ) return hipErrorNotSupported;
-  const long long threads = (long long)p.rowsA * (p.rowsB >> 2) * 8;
-  const unsigned blocks = (unsigned)((threads + 255) / 256);
+  const unsigned blocks = (unsigned)(((p.rowsA + 3) / 4) * ((p.rowsB + 31) / 32));
   if (p.KW <= 32)
     hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, 1>), dim3(blocks), dim3(256), 0, stream, p);
   else
