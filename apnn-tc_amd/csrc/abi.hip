@@ -118,6 +118,14 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   return nullptr;
 }
 
+// what the register-only kernel (valu_direct_kernel.h) handles
+bool direct_kernel_serves(const KParams &p) {
+  if ((p.rowsB & 3) != 0 || (p.KW & 3) != 0) return false;
+  if (p.epi == APNN_EPI_INT32) return true;
+  return (p.rowsB & 31) == 0 && p.pool == APNN_POOL_NONE && p.resid == nullptr && p.save_acc == nullptr &&
+         p.resid_planes == nullptr;
+}
+
 typedef hipError_t (*patch_fn)(int, const KParams &, hipStream_t);
 patch_fn patch_conv_fn(int xb, int wb) {
   if (xb == 2 && wb == 1) return apnn::patch_conv_2_1_x;
@@ -295,12 +303,11 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
-  const bool direct_ok = d->epi.mode == APNN_EPI_INT32 && fn != apnn::valu_gemm_any_x && (p.rowsB & 3) == 0 &&
-                         p.KW <= 64;
-  if (tile_pin == apnn::TILE_DIRECT + 1)  // register-only kernel: int32 output, K <= 2048
+  const bool direct_ok = fn != apnn::valu_gemm_any_x && direct_kernel_serves(p);
+  if (tile_pin == apnn::TILE_DIRECT + 1)  // register-only kernel
     return direct_ok ? from_hip(fn(4, apnn::TILE_DIRECT, p, stream)) : APNN_EUNSUPPORTED;
   // small, latency-bound problems (the M = 64 sweep): one round of loads, no LDS, no barrier
-  if (tile_pin == 0 && direct_ok && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
+  if (tile_pin == 0 && direct_ok && p.KW <= 64 && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
     return from_hip(fn(4, apnn::TILE_DIRECT, p, stream));
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
   return (int)fn(4, tile, p, stream);
@@ -358,6 +365,18 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;
+  // A filter that spans the whole stored input map (fully connected layer): every output pixel is one
+  // image, whose im2col row is the image itself -- a plain GEMM over rows of KW words.  With few
+  // outputs (small batch) the layer streams its weights; the register-only kernel serves it.
+  const bool fc_shape = Ho == 1 && Wo == 1 && p.pad == 0 && d->R == p.Hs && d->S == p.Ws;
+  {
+    valu_fn vf = valu_conv_fn(d->xb, d->wb);
+    const bool fc_direct_ok = fc_shape && vf != nullptr && vf != apnn::valu_conv_any_x && direct_kernel_serves(p);
+    if (path == APNN_PATH_VALU && tile_pin == apnn::TILE_DIRECT + 1)
+      return fc_direct_ok ? from_hip(vf(vw, apnn::TILE_DIRECT, p, stream)) : APNN_EUNSUPPORTED;
+    if (path == APNN_PATH_AUTO && tile_pin == 0 && fc_direct_ok && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
+      return from_hip(vf(vw, apnn::TILE_DIRECT, p, stream));
+  }
   if (path == APNN_PATH_MFMA_PATCH || path == APNN_PATH_AUTO) {
     patch_fn pf = patch_conv_fn(d->xb, d->wb);
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);

@@ -14,6 +14,8 @@ namespace apnn {
 
 #if INST_CONV
 hipError_t APNN_CAT(valu_conv_, INST_PA, INST_PB, x)(int vw, int tile, const KParams &p, hipStream_t s) {
+  // fully connected layer (filter spans the input map): rows of A are whole images, a plain GEMM
+  if (tile == TILE_DIRECT) return launch_valu_direct<INST_PA, INST_PB, true>(p, s);
   switch (vw) {
     case 4: return launch_valu_tile<INST_PA, INST_PB, 4, true>(tile, p, s);
     case 2: return launch_valu_tile<INST_PA, INST_PB, 2, true>(tile, p, s);
@@ -23,7 +25,7 @@ hipError_t APNN_CAT(valu_conv_, INST_PA, INST_PB, x)(int vw, int tile, const KPa
 #else
 hipError_t APNN_CAT(valu_gemm_, INST_PA, INST_PB, x)(int vw, int tile, const KParams &p, hipStream_t s) {
   (void)vw;  // GEMM rows are whole int4 words (K % 128 == 0)
-  if (tile == TILE_DIRECT) return launch_valu_direct<INST_PA, INST_PB>(p, s);
+  if (tile == TILE_DIRECT) return launch_valu_direct<INST_PA, INST_PB, false>(p, s);
   return launch_valu_tile<INST_PA, INST_PB, 4, false>(tile, p, s);
 }
 #endif

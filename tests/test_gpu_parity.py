@@ -624,7 +624,7 @@ def test_quantize_pack(G, bits, rows, C, cpad):
 
 @pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("wb,xb", COMBOS)
-@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (50, 36, 128), (1, 4, 2048), (64, 128, 1536), (7, 260, 640)])
+@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (50, 36, 128), (1, 4, 2048), (64, 128, 1536), (7, 260, 640), (8, 64, 9216)])
 def test_gemm_register_only_kernel(G, M, N, K, wb, xb, sym):
     """The latency-oriented GEMM kernel (eight lanes split K for four outputs), pinned as VALU tile 4."""
     rng = np.random.default_rng(7000 + M + N + K + 10 * wb + xb + sym)
@@ -636,12 +636,54 @@ def test_gemm_register_only_kernel(G, M, N, K, wb, xb, sym):
 
 def test_gemm_register_only_kernel_limits(G):
     rng = np.random.default_rng(7100)
-    W = O.random_planes(rng, 1, 8, 4096 // 32)
-    X = O.random_planes(rng, 2, 8, 4096 // 32)
-    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):     # K > 2048
-        G.run_gemm(W, X, 8, 8, 4096, 1, 2, path=1, tile=4)
     W = O.random_planes(rng, 1, 8, 4)
     X = O.random_planes(rng, 2, 6, 4)
     with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):     # N % 4 != 0
         G.run_gemm(W, X, 8, 6, 128, 1, 2, path=1, tile=4)
     assert np.array_equal(G.run_gemm(W, X, 8, 6, 128, 1, 2).reshape(8, 6), O.gemm(W, X, 8, 6, 128, 1, 2))
+    X = O.random_planes(rng, 2, 32, 4)
+    resid = G.to_dev(np.zeros((8, 32), np.int32))
+    d_thr = G.to_dev(np.zeros((32, 3), np.int32))
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):     # no residual input in this kernel
+        G.run_gemm(W, X, 8, 32, 128, 1, 2, epi=G.epilogue(mode=G.A.EPI_BN, out_bits=2, thr=d_thr, resid=resid),
+                   path=1, tile=4)
+
+
+@pytest.mark.parametrize("sym", [0, 1])
+@pytest.mark.parametrize("wb,xb,ob", [(1, 2, 2), (1, 4, 4), (2, 2, 1), (1, 3, 3)])
+@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (9, 96, 4096), (5, 32, 384)])
+def test_gemm_register_only_kernel_packed(G, M, N, K, wb, xb, ob, sym):
+    rng = np.random.default_rng(7200 + M + N + 10 * wb + xb + sym)
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, wb, xb, sym_w=sym)
+    thr = np.sort(rng.integers(int(acc.min()), int(acc.max()) + 1, size=(N, 2 ** ob - 1)), axis=1).astype(np.int32)
+    flip = rng.integers(0, 2, size=N).astype(np.uint8)
+    thr[flip == 1] = -thr[flip == 1, ::-1]
+    d_thr, d_flip = G.to_dev(thr), G.to_dev(flip)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, flip=d_flip)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, epi=epi, path=1, tile=4).view(np.uint32).reshape(ob, M, N // 32)
+    assert np.array_equal(got, O.lowbits_pack(O.bn_quantize(acc, None, thr, flip, ob), M, N, ob))
+    epi = G.epilogue(mode=G.A.EPI_LOWBITS, out_bits=ob)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, epi=epi, path=1, tile=4).view(np.uint32).reshape(ob, M, N // 32)
+    assert np.array_equal(got, O.lowbits_pack(acc & (2 ** ob - 1), M, N, ob))
+
+
+@pytest.mark.parametrize("path,tile", [(1, 4), (0, None), (2, None)])
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("batch,H,Wd,C,cout", [(8, 6, 6, 256, 512), (3, 7, 7, 128, 96), (16, 1, 1, 1024, 256)])
+def test_fully_connected_layer_as_convolution(G, batch, H, Wd, C, cout, wb, xb, path, tile):
+    """Filter spans the feature map: AUTO / the pinned register-only kernel treat it as a GEMM over whole
+    images; int32 and quantized packed output against the oracle convolution."""
+    rng = np.random.default_rng(7300 + batch + C + 10 * wb + xb)
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, cout * H * Wd, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=H, S=Wd, stride=1, pad=0, halo=0, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw).reshape(batch, cout)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, path=path, tile=tile, **kw).reshape(batch, cout)
+    assert np.array_equal(got, acc)
+    thr = np.sort(rng.integers(int(acc.min()), int(acc.max()) + 1, size=(cout, 3)), axis=1).astype(np.int32)
+    d_thr = G.to_dev(thr)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=2, thr=d_thr)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(2, batch, cout // 32)
+    assert np.array_equal(got, O.lowbits_pack(O.bn_quantize(acc, None, thr, None, 2), batch, cout, 2))
