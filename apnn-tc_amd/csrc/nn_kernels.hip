@@ -692,54 +692,64 @@ __global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restr
 }
 
 // ---- int8 classifier: out[b][n] = scale[n] * sum_k X[b][k] * Wt[n][k] + bias[n] -----------------
-// One wave per (output feature n, group of four batch rows): lanes stride over K in dwords
-// (v_dot4_i32_i8 on four int8 pairs), each weight dword is used for the four rows, then a wave64
-// butterfly reduction.  K % 4 != 0 (or unaligned rows) falls back to byte loads.
+// One wave per (group of NN output features, group of four batch rows): lanes stride over K in dwords
+// (v_dot4_i32_i8 on four int8 pairs), every operand dword is used NN or four times, then wave64
+// butterfly reductions.  K % 4 != 0 (or unaligned rows) falls back to byte loads.
+// NN output features x 4 batch rows per wave (NN = 4 when the batch is large enough to make operand
+// re-reads the cost, else 1: more waves for small batches).
+template <int NN>
 __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                     const float *__restrict__ scale, const float *__restrict__ bias,
                                                     float *__restrict__ out, int32_t *__restrict__ acc_out, int Bn,
                                                     int N, int K, int vec_ok) {
   const int lane = threadIdx.x & 63;
-  const int bgroups = (Bn + 3) >> 2;
+  const int bgroups = (Bn + 3) >> 2, ngroups = (N + NN - 1) / NN;
   const long long wid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (wid >= (long long)N * bgroups) return;
-  const int n = (int)(wid % N);
-  const int8_t *w = Wt + (long long)n * K;
-  const float sc = scale[n], bi = bias[n];
-  {
-    const int b0 = (int)(wid / N) * 4;
-    int acc[4] = {0, 0, 0, 0};
-    if (vec_ok) {
-      const int *w4 = reinterpret_cast<const int *>(w);
-      for (int k4 = lane; k4 < (K >> 2); k4 += 64) {
-        const int wv = w4[k4];
+  if (wid >= (long long)ngroups * bgroups) return;
+  const int n0 = (int)(wid % ngroups) * NN;
+  const int b0 = (int)(wid / ngroups) * 4;
+  int acc[NN][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (b0 + j < Bn) {
-            const int xv = reinterpret_cast<const int *>(X + (long long)(b0 + j) * K)[k4];
-            acc[j] = __builtin_amdgcn_sdot4(xv, wv, acc[j], false);
-          }
-        }
-      }
-    } else {
-      for (int k = lane; k < K; k += 64) {
-        const int wv = w[k];
+  for (int i = 0; i < NN; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0;
+  if (vec_ok) {
+    for (int k4 = lane; k4 < (K >> 2); k4 += 64) {
+      int wv[NN], xv[4];
+#pragma unroll
+      for (int i = 0; i < NN; ++i)
+        wv[i] = n0 + i < N ? reinterpret_cast<const int *>(Wt + (long long)(n0 + i) * K)[k4] : 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        xv[j] = b0 + j < Bn ? reinterpret_cast<const int *>(X + (long long)(b0 + j) * K)[k4] : 0;
+#pragma unroll
+      for (int i = 0; i < NN; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_sdot4(xv[j], wv[i], acc[i][j], false);
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) {
+#pragma unroll
+      for (int i = 0; i < NN; ++i) {
+        const int wv = n0 + i < N ? (int)Wt[(long long)(n0 + i) * K + k] : 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          if (b0 + j < Bn) acc[j] += (int)X[(long long)(b0 + j) * K + k] * wv;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) acc[j] += __shfl_xor(acc[j], off, 64);
-      if (lane == 0 && b0 + j < Bn) {
-        const long long o = (long long)(b0 + j) * N + n;
-        if (acc_out != nullptr) acc_out[o] = acc[j];
-        out[o] = (float)acc[j] * sc + bi;
+          if (b0 + j < Bn) acc[i][j] += (int)X[(long long)(b0 + j) * K + k] * wv;
       }
     }
   }
+#pragma unroll
+  for (int i = 0; i < NN; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) acc[i][j] += __shfl_xor(acc[i][j], off, 64);
+      if (lane == 0 && b0 + j < Bn && n0 + i < N) {
+        const long long o = (long long)(b0 + j) * N + n0 + i;
+        if (acc_out != nullptr) acc_out[o] = acc[i][j];
+        out[o] = (float)acc[i][j] * scale[n0 + i] + bias[n0 + i];
+      }
+    }
 }
 
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,
@@ -864,9 +874,15 @@ hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows
 hipError_t launch_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
                         int32_t *acc_out, int Bn, int N, int K, hipStream_t s) {
   const int vec_ok = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Wt)) & 3u) == 0;
-  const long long waves = (long long)N * ((Bn + 3) / 4);
-  hipLaunchKernelGGL(fc_i8_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out,
-                     acc_out, Bn, N, K, vec_ok);
+  if ((long long)N * ((Bn + 3) / 4) >= 8192) {  // plenty of waves: four features per wave cut the re-reads of X
+    const long long waves = (long long)((N + 3) / 4) * ((Bn + 3) / 4);
+    hipLaunchKernelGGL(fc_i8_kernel<4>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out,
+                       acc_out, Bn, N, K, vec_ok);
+  } else {
+    const long long waves = (long long)N * ((Bn + 3) / 4);
+    hipLaunchKernelGGL(fc_i8_kernel<1>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out,
+                       acc_out, Bn, N, K, vec_ok);
+  }
   return hipGetLastError();
 }
 
