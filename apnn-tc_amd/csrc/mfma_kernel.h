@@ -792,12 +792,13 @@ constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB,
   return stage > slab ? stage : slab;
 }
 
-// OCC_WANTED work-groups per compute unit if the LDS budget (160 KiB) allows it, else one
+// OCC_WANTED work-groups per compute unit, or as many as the LDS budget (160 KiB) allows
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
   constexpr size_t smem_bytes = mfma_smem_bytes(PA, PB, FA, FB, WA, WB, CONV);
-  constexpr int OCC = (OCC_WANTED > 1 && smem_bytes * OCC_WANTED <= 160 * 1024) ? OCC_WANTED : 1;
+  constexpr int OCC_FIT = (int)((160 * 1024) / smem_bytes);
+  constexpr int OCC = OCC_FIT < 1 ? 1 : (OCC_FIT < OCC_WANTED ? OCC_FIT : OCC_WANTED);
   static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
   auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>;
   if (smem_bytes > 64 * 1024) {
