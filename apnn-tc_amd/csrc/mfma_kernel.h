@@ -492,9 +492,10 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
   // k-words (32 elements each) per staged chunk.  The convolution kernels whose waves tile the output
   // (64x64 and 128x64 per work-group with 128-bit loads, i.e. at least 128 stored channels; larger tiles
-  // and the short reductions of narrow layers measure no gain) stage 16: their per-chunk work (im2col addressing, LDS staging, barrier) is a large share of a
+  // and the short reductions of narrow layers measure no gain) stage 16; the split-K tiles, used for
+  // few outputs over a long K where every chunk iteration is a latency chain, stage 32: their per-chunk work (im2col addressing, LDS staging, barrier) is a large share of a
   // short K loop, and k-steps past the end of K are skipped, so a longer chunk wastes nothing.
-  constexpr int KC = (CONV && KS == 1 && FA * FB <= 2 && VW == 4) ? 16 : 8;
+  constexpr int KC = KS > 1 ? 32 : (CONV && FA * FB <= 2 && VW == 4) ? 16 : 8;
   constexpr int LD = KC + 1;         // odd row pitch: 32 rows hit 32 different banks
   constexpr int KQ = KC / VW;
   constexpr int UA = TA * KQ, UB = TB * KQ;
@@ -787,7 +788,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
 }
 
 constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
-  const size_t ld = (conv && WA * WB == 4 && FA * FB <= 2 && vw == 4) ? 17 : 9;  // KC + 1, see the kernel
+  const size_t ld = WA * WB == 1 ? 33 : (conv && FA * FB <= 2 && vw == 4) ? 17 : 9;  // KC + 1, see the kernel
   const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
   const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
   return stage > slab ? stage : slab;
