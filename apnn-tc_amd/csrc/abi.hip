@@ -216,6 +216,14 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
     return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
   }
   if (conv && vw == 1) return (ntiles(2) >= cus / 2 || KW < 16) ? 2 : 4;  // 32-bit loads: two tiles built
+  // Few outputs over a long reduction (batch-1 / batch-8 layers, 7x7 maps): the split-K tiles give
+  // every 32x32 (32x64) block a work-group of its own and the four waves share K.  Measured
+  // cross-overs on ResNet18 / 16x16 benchmark shapes.
+  if (conv) {
+    const long long nb32 = ntiles(4);
+    if (KW >= 32 && nb32 <= 640) return 4;
+    if (KW >= 128 && nb32 <= 2560) return 5;
+  }
   if (rowsB <= 64 && ntiles(3) >= cus) return 3;
   if (rowsB > 64) {
     const int big = conv ? 7 : 6;
@@ -240,13 +248,18 @@ int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, i
 }
 
 // AUTO: the matrix-core path pays off once there are enough 32x32 blocks to fill the chip (measured
-// cross-over: about 256x256 outputs, at any reduction length); smaller, latency-bound problems stay on
-// the VALU path, whose 16x16 tiles spread them over more compute units.
-bool auto_prefers_mfma(const KParams &p) { return (long long)p.rowsA * p.rowsB >= 256LL * 256; }
+// cross-over: about 256x256 outputs at any reduction length, 128x128 when K is at least 1024 bits and
+// the split-K tile applies); smaller, latency-bound problems stay on the VALU path, whose 16x16 tiles
+// spread them over more compute units.
+bool auto_prefers_mfma(const KParams &p) {
+  const long long outputs = (long long)p.rowsA * p.rowsB;
+  return outputs >= 256LL * 256 || (outputs >= 128LL * 128 && p.KW >= 32);  // long K: split-K matrix-core tile
+}
 // GEMM at exactly the cross-over size with a short reduction (64 x 1024 outputs over 1024 bits): both
 // paths sit on the launch floor and the VALU tile measures a few percent faster.
 bool auto_prefers_mfma_gemm(const KParams &p) {
-  return auto_prefers_mfma(p) && ((long long)p.rowsA * p.rowsB > 256LL * 256 || p.KW > 32);
+  const long long outputs = (long long)p.rowsA * p.rowsB;
+  return outputs > 256LL * 256 || (outputs == 256LL * 256 && p.KW > 32);
 }
 
 valu_fn valu_gemm_fn(int wb, int xb) {
