@@ -234,7 +234,9 @@ def main():
             convs = []
             for (w_, a_) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
                 for batch in (1, 16):
-                    for C in (128, 256, 512, 1024) if (w_, a_) == (1, 2) else (512, 1024):
+                    # w1a2 at batch 1: the reference's published list (README.md:160-167)
+                    for C in ((128, 256, 384, 512, 640, 768, 896, 1024) if batch == 1 else (128, 256, 512, 1024)) \
+                            if (w_, a_) == (1, 2) else (512, 1024):
                         for fused in (False, True):
                             t = time_conv(batch, C, w_, a_, fused, 10, 200 if batch == 1 else 50)
                             t["shape"] = "w%da%d 3x3 16x16 b%d Cin=Cout=%d %s" % (
