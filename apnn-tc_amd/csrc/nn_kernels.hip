@@ -355,18 +355,34 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   const int co0 = blockIdx.y * 64;
   const int SC = S * C;
 
-  // filter block -> LDS, one 16-byte half per task (its byte loads are independent of each other)
-  for (int task = tid; task < 64 * nks * 2; task += 256) {
-    const int col = task / (nks * 2), hh = task - col * (nks * 2);
-    const int r = hh / HPR, hq = hh - r * HPR;
-    const int co = co0 + col;
-    const int nvalid = (co < COUT && r < R) ? min(max(SC - hq * 16, 0), 16) : 0;
-    const int8_t *src = Wt + ((long long)co * R + r) * SC + hq * 16;
-    uint32_t w[4] = {0, 0, 0, 0};
+  // filter block -> LDS, one 16-byte half per task.  Four tasks per thread are in flight at a time:
+  // all their byte loads are issued before the first LDS store, so the block costs one or two memory
+  // round trips instead of one per task.
+  const int ntasks = 64 * nks * 2;
+  for (int t0 = 0; t0 < ntasks; t0 += 4 * 256) {
+    uint32_t w[4][4];
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      if (i < nvalid) w[i >> 2] |= (uint32_t)(uint8_t)src[i] << (8 * (i & 3));
-    *reinterpret_cast<uint4 *>(wl + col * KPL + hh * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    for (int u = 0; u < 4; ++u) {
+      const int task = t0 + u * 256 + tid;
+      const int col = task / (nks * 2), hh = task - col * (nks * 2);
+      const int r = hh / HPR, hq = hh - r * HPR;
+      const int co = co0 + col;
+      const int nvalid = (task < ntasks && co < COUT && r < R) ? min(max(SC - hq * 16, 0), 16) : 0;
+      const int8_t *src = Wt + ((long long)co * R + r) * SC + hq * 16;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[u][q] = 0;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (i < nvalid) w[u][i >> 2] |= (uint32_t)(uint8_t)src[i] << (8 * (i & 3));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int task = t0 + u * 256 + tid;
+      if (task < ntasks) {
+        const int col = task / (nks * 2), hh = task - col * (nks * 2);
+        *reinterpret_cast<uint4 *>(wl + col * KPL + hh * 16) = make_uint4(w[u][0], w[u][1], w[u][2], w[u][3]);
+      }
+    }
   }
   __syncthreads();
 
