@@ -326,7 +326,8 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   return (int)fn(4, tile, p, stream);
 }
 
-int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
+// validation + kernel-side description of a convolution
+int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   if (d == nullptr) return APNN_ENULL;
   int rc;
   if ((rc = check_dev_ptr(d->W)) || (rc = check_dev_ptr(d->X)) || (rc = check_dev_ptr(d->O))) return rc;
@@ -335,7 +336,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (d->R <= 0 || d->S <= 0 || d->stride <= 0 || d->pad < 0) return APNN_EINVAL;
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
-  const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
+  const int path = d->path & 0xff;
   if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_PATCH))
     return APNN_EINVAL;
   if (d->H + 2 * d->pad < d->R || d->Wd + 2 * d->pad < d->S) return APNN_EINVAL;
@@ -349,7 +350,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   // a chunk of 4 words must not straddle two taps when 128-bit loads are used
   const int vw = (C32 % 4 == 0) ? 4 : (C32 % 2 == 0) ? 2 : 1;
 
-  KParams p{};
+  p = KParams{};
   p.A = static_cast<const uint32_t *>(d->X);
   p.B = static_cast<const uint32_t *>(d->W);
   p.rowsA = (int)pixels;
@@ -372,12 +373,21 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   p.wmax = (1 << d->wb) - 1;
   fill_epilogue(p, d->epi, d->O, p.pool_order ? pixels / 4 : pixels);
 
-  int tile;
   p.planesA = d->xb;
   p.planesB = d->wb;
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;
+  *vw_out = vw;
+  return APNN_OK;
+}
+
+int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
+  KParams p{};
+  int vw = 1, rc, tile;
+  if ((rc = build_conv_params(d, p, &vw))) return rc;
+  const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
+  const int Ho = p.Ho, Wo = p.Wo;
   // A filter that spans the whole stored input map (fully connected layer): every output pixel is one
   // image, whose im2col row is the image itself -- a plain GEMM over rows of KW words.  With few
   // outputs (small batch) the layer streams its weights; the register-only kernel serves it.
@@ -415,6 +425,43 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   if (fn == nullptr) return APNN_EUNSUPPORTED;
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
   return (int)fn(vw, tile, p, stream);
+}
+
+// Same input, same output grid, same precision / epilogue mode; see apnn_conv_pair in apnn_tc.h.
+int run_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, hipStream_t stream) {
+  KParams pa{}, pb{};
+  int vwa = 1, vwb = 1, rc;
+  if ((rc = build_conv_params(a, pa, &vwa)) || (rc = build_conv_params(b, pb, &vwb))) return rc;
+  const bool same = a->X == b->X && a->batch == b->batch && a->H == b->H && a->Wd == b->Wd &&
+                    a->cin_pad == b->cin_pad && a->COUT == b->COUT && a->stride == b->stride && a->halo == b->halo &&
+                    a->wb == b->wb && a->xb == b->xb && a->weight_mode == b->weight_mode && pa.Ho == pb.Ho &&
+                    pa.Wo == pb.Wo && pa.Hs == pb.Hs && pa.Ws == pb.Ws;
+  if (!same) return APNN_EINVAL;
+  auto plain_bn = [](const apnn_epilogue &e) {
+    return e.mode == APNN_EPI_BN && e.pool == APNN_POOL_NONE && e.residual == nullptr && e.save_acc == nullptr &&
+           e.residual_planes == nullptr;
+  };
+  valu_fn fn = mfma_conv_fn(a->xb, a->wb, false);
+  const bool fusable = fn != nullptr && plain_bn(a->epi) && plain_bn(b->epi) && a->epi.out_bits == b->epi.out_bits &&
+                       (a->path & 0xffff) == APNN_PATH_AUTO && (b->path & 0xffff) == APNN_PATH_AUTO &&
+                       auto_prefers_mfma(pa) && a->O != b->O;
+  if (!fusable) {
+    if ((rc = run_conv(a, stream))) return rc;
+    return run_conv(b, stream);
+  }
+  // tile for the larger of the two problems, evaluated for twice the number of work-groups
+  int tile = choose_mfma_tile(2 * pa.rowsA, pa.rowsB, pa.KW, true, vwa, false);
+  pa.pair_tiles = 1;  // flag; the launcher fills in the tile count
+  pa.B2 = pb.B;
+  pa.KW2 = pb.KW;
+  pa.S2 = pb.S;
+  pa.pad2 = pb.pad;
+  pa.magicS2 = pb.magicS;
+  pa.planeB2 = pb.planeB;
+  pa.thr2 = pb.thr;
+  pa.flip2 = pb.flip;
+  pa.out2 = pb.out;
+  return from_hip(fn(vwa, tile, pa, stream));
 }
 
 int named_gemm(int want_wb, int want_xb, int mode, const void *W, const void *X, int *D, int M, int N, int K,
@@ -507,6 +554,9 @@ APNN_DEF_CONV(APConv_w2a2_pack_pool, 2, 2, APNN_EPI_LOWBITS, APNN_POOL_AVG2X2)
 
 int apnn_gemm(const apnn_gemm_desc *d, apnn_stream_t s) { return run_gemm(d, static_cast<hipStream_t>(s)); }
 int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s) { return run_conv(d, static_cast<hipStream_t>(s)); }
+int apnn_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, apnn_stream_t s) {
+  return run_conv_pair(a, b, static_cast<hipStream_t>(s));
+}
 
 int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
                    apnn_stream_t s) {

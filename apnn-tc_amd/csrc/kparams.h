@@ -37,6 +37,19 @@ struct KParams {
   // exact quotients for dividends below d + 1024
   uint32_t magicGW, magicGH, magicPW, magicPH;
 
+  // Paired launch (matrix-core convolution kernels only): work-groups pair_tiles .. 2*pair_tiles-1
+  // compute a second convolution on the same input and output grid (same A, rows, columns, stride,
+  // precisions, epilogue mode) that differs in filter, filter size, padding, thresholds and output:
+  // the two branches of a residual block's entry (3x3 convolution and 1x1 downsample) in one launch.
+  int pair_tiles;            // 0: single problem
+  const uint32_t *B2;
+  int KW2, S2, pad2;
+  uint32_t magicS2;
+  long long planeB2;
+  const int32_t *thr2;
+  const uint8_t *flip2;
+  void *out2;
+
   int sym;                   // symmetric weights: result = 2*raw - wmax * (activation row sum)
   int wmax;                  // 2^wb - 1
 

@@ -477,7 +477,22 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
 
 
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
-__global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
+__global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
+  // paired launch: the second half of the grid works on the second problem (see KParams)
+  KParams p = pk;
+  int bid = blockIdx.x;
+  if (CONV && pk.pair_tiles > 0 && bid >= pk.pair_tiles) {
+    bid -= pk.pair_tiles;
+    p.B = pk.B2;
+    p.KW = pk.KW2;
+    p.S = pk.S2;
+    p.pad = pk.pad2;
+    p.magicS = pk.magicS2;
+    p.planeB = pk.planeB2;
+    p.thr = pk.thr2;
+    p.flip = pk.flip2;
+    p.out = pk.out2;
+  }
   // four waves per work-group: WA x WB of them tile the output, the remaining factor KS splits K
   static_assert(WA * WB == 4 || WA * WB == 1, "waves tile the output or all split K");
   constexpr int KS = 4 / (WA * WB);
@@ -510,8 +525,8 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams p) {
   const int wa = KS > 1 ? 0 : wave / WB, wb = KS > 1 ? 0 : wave % WB;
 
   const int tilesB = (p.rowsB + TB - 1) / TB;
-  const int a0 = (blockIdx.x / tilesB) * TA;
-  const int b0 = (blockIdx.x % tilesB) * TB;
+  const int a0 = (bid / tilesB) * TA;
+  const int b0 = (bid % tilesB) * TB;
 
   // ---- staging bookkeeping (same scheme as the VALU kernel) ----------------------------------
   int a_row[NIA], a_kq[NIA];
@@ -813,7 +828,9 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
     }
   }
   const long long tiles = (long long)((p.rowsA + TA - 1) / TA) * ((p.rowsB + TB - 1) / TB);
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), smem_bytes, stream, p);
+  KParams q = p;
+  if (p.pair_tiles != 0) q.pair_tiles = (int)tiles;  // the host only flags a pair; the tile count is known here
+  hipLaunchKernelGGL(kern, dim3((unsigned)(q.pair_tiles != 0 ? 2 * tiles : tiles)), dim3(256), smem_bytes, stream, q);
   return hipGetLastError();
 }
 

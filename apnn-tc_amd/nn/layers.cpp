@@ -182,7 +182,7 @@ int Conv128LayerParam::initialize(Rng &rng, const uint32_t *prev_layer_gpu, cons
   return 0;
 }
 
-int Conv_new_global(Conv128LayerParam *p, hipStream_t stream) {
+static apnn_conv_desc conv_desc_of(const Conv128LayerParam *p) {
   apnn_conv_desc d{};
   d.W = p->filter_gpu.get();
   d.X = p->input_gpu;
@@ -208,7 +208,17 @@ int Conv_new_global(Conv128LayerParam *p, hipStream_t stream) {
   d.epi.residual_bits = p->a_bit;
   d.epi.residual_scale = p->residual_scale;
   d.path = p->path;
+  return d;
+}
+
+int Conv_new_global(Conv128LayerParam *p, hipStream_t stream) {
+  const apnn_conv_desc d = conv_desc_of(p);
   return apnn_conv(&d, stream);
+}
+
+int Conv_pair_global(Conv128LayerParam *main_branch, Conv128LayerParam *shortcut_branch, hipStream_t stream) {
+  const apnn_conv_desc a = conv_desc_of(main_branch), b = conv_desc_of(shortcut_branch);
+  return apnn_conv_pair(&a, &b, stream);
 }
 
 int Conv128LayerParam::forward(hipStream_t stream) { return Conv_new_global(this, stream); }
@@ -364,8 +374,18 @@ int Network::forward(const uint8_t *images, float *logits, hipStream_t stream) {
   if (images == nullptr || logits == nullptr) return APNN_ENULL;
   first->set_input_gpu(images);
   last->set_output_gpu(logits);
-  for (auto &l : layers) {
-    const int rc = l->forward(stream);
+  for (size_t i = 0; i < layers.size(); ++i) {
+    // a residual block's first convolution and the downsample convolution listed right after it read
+    // the same input: one paired launch
+    if (i + 1 < layers.size() && layers[i + 1]->pairs_with_previous) {
+      auto *a = static_cast<Conv128LayerParam *>(layers[i].get());
+      auto *b = static_cast<Conv128LayerParam *>(layers[i + 1].get());
+      const int rc = Conv_pair_global(a, b, stream);
+      if (rc != 0) return rc;
+      ++i;
+      continue;
+    }
+    const int rc = layers[i]->forward(stream);
     if (rc != 0) return rc;
   }
   return 0;

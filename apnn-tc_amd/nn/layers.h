@@ -65,6 +65,9 @@ class Layer {
   virtual int forward(hipStream_t stream) = 0;
   virtual void describe(apnn_layer_desc *d) const = 0;
   virtual const uint32_t *get_output_gpu() const { return nullptr; }
+  // set on a Conv128LayerParam that reads the same input as the Conv128LayerParam listed before it
+  // (the 1x1 downsample convolution of a residual block): the network launches the two as a pair
+  bool pairs_with_previous = false;
 };
 
 // First layer: int8 convolution on uint8 pixels (zero point 128), thresholds -> a-bit codes,
@@ -168,6 +171,8 @@ class Out128LayerParam : public Layer {
 // kernel call.  The reference launches a __global__ wrapper around a __device__ kernel; here the
 // wrapper is a host function that enqueues on `stream`.
 int Conv_new_global(Conv128LayerParam *p, hipStream_t stream);
+// both branches of a residual block's entry (3x3 convolution, 1x1 downsample) in one launch
+int Conv_pair_global(Conv128LayerParam *main_branch, Conv128LayerParam *shortcut_branch, hipStream_t stream);
 int FC_new_global(Fc128LayerParam *p, hipStream_t stream);
 int Output_new_global(Out128LayerParam *p, hipStream_t stream);
 

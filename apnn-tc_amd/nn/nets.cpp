@@ -119,6 +119,7 @@ std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path) {
         snprintf(nm, sizeof nm, "L%dB%dDS", stage + 1, blk + 1);
         auto *ds = add(*net, new Conv128LayerParam(nm, h, w, 1, 1, cin, ch, batch, stride, stride, false));
         if (ds->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+        ds->pairs_with_previous = true;  // same input as c1: launched together
         shortcut = ds->get_output_gpu();
         shortcut_index = (int)net->layers.size() - 1;
       }

@@ -179,6 +179,16 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
 
 /* ---- layers on either side of the low-bit path ------------------------------------------------ */
 
+/* Two convolutions of the same input onto the same output grid in one launch: the entry of a residual
+ * block, where the 3x3 convolution of the main branch and the 1x1 downsample convolution of the
+ * shortcut both read the block input (no counterpart in the reference, whose ResNet18 has no downsample
+ * convolution, APNN-TC-nn/src/resnet18.cu:40-142).  a and b must agree in X, batch, H, Wd, cin_pad, COUT,
+ * stride, halo, wb, xb, weight_mode and output size, and both use APNN_EPI_BN with the same out_bits and no
+ * pooling / residual inputs; filter, filter size, padding, thresholds, flip and output differ.  When the
+ * pair cannot share a matrix-core kernel the two are launched one after the other: the result is the
+ * same either way. */
+int apnn_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, apnn_stream_t s);
+
 /* Float tensor -> bit-planes in one pass: the affine quantizer of Quantize_val
  * (APNN-TC-nn/src/kernel.cuh:29-44; the reference computes the code but its store is commented out)
  *     code = min(2^bits - 1, rint(((clip(x, min_v, max_v) - min_v) * 2^bits * 1.0f) / (max_v - min_v)))

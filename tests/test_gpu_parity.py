@@ -687,3 +687,41 @@ def test_fully_connected_layer_as_convolution(G, batch, H, Wd, C, cout, wb, xb, 
     epi = G.epilogue(mode=G.A.EPI_BN, out_bits=2, thr=d_thr)
     got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(2, batch, cout // 32)
     assert np.array_equal(got, O.lowbits_pack(O.bn_quantize(acc, None, thr, None, 2), batch, cout, 2))
+
+
+@pytest.mark.parametrize("batch,H,C,cout", [(8, 28, 128, 256), (64, 14, 256, 512), (2, 56, 64, 128), (1, 8, 128, 64)])
+@pytest.mark.parametrize("wb,xb", [(1, 2), (2, 2), (1, 4)])
+def test_conv_pair_residual_block_entry(G, batch, H, C, cout, wb, xb):
+    """3x3 stride-2 convolution and 1x1 stride-2 downsample of the same input in one call: each output
+    equals the convolution launched on its own (and the oracle)."""
+    rng = np.random.default_rng(8000 + batch + H + 10 * wb + xb)
+    X = O.random_planes(rng, xb, batch * H * H, C // 32)
+    W3 = O.random_planes(rng, wb, cout * 9, C // 32)
+    W1 = O.random_planes(rng, wb, cout, C // 32)
+    k3 = dict(batch=batch, H=H, W=H, cout=cout, R=3, S=3, stride=2, pad=1, halo=0, wb=wb, xb=xb)
+    k1 = dict(batch=batch, H=H, W=H, cout=cout, R=1, S=1, stride=2, pad=0, halo=0, wb=wb, xb=xb)
+    acc3 = O.conv(W3, X, cwords=C // 32, sym_w=1, nthreads=8, **k3).reshape(-1, cout)
+    acc1 = O.conv(W1, X, cwords=C // 32, sym_w=1, nthreads=8, **k1).reshape(-1, cout)
+    rows = acc3.shape[0]
+    assert acc1.shape[0] == rows
+    nt = 2 ** xb - 1
+    thr3 = np.sort(rng.integers(int(acc3.min()), int(acc3.max()) + 1, size=(cout, nt)), axis=1).astype(np.int32)
+    thr1 = np.sort(rng.integers(int(acc1.min()), int(acc1.max()) + 1, size=(cout, nt)), axis=1).astype(np.int32)
+    dX, dW3, dW1, dT3, dT1 = G.to_dev(X), G.to_dev(W3), G.to_dev(W1), G.to_dev(thr3), G.to_dev(thr1)
+    words = xb * rows * cout // 32
+    o3, o1 = G.dev_empty_i32(words, fill=-7), G.dev_empty_i32(words, fill=-7)
+    A = G.A
+    def desc(Wd_, out, R, pad, thr):
+        return A.ConvDesc(W=Wd_.data_ptr(), X=dX.data_ptr(), O=out.data_ptr(), batch=batch, H=H, Wd=H, cin_pad=C,
+                          COUT=cout, R=R, S=R, stride=2, pad=pad, halo=0, wb=wb, xb=xb, weight_mode=A.WEIGHT_SYMMETRIC,
+                          epi=G.epilogue(mode=A.EPI_BN, out_bits=xb, thr=thr), path=A.PATH_AUTO)
+    da, db = desc(dW3, o3, 3, 1, dT3), desc(dW1, o1, 1, 0, dT1)
+    A.check(A.lib().apnn_conv_pair(ctypes.byref(da), ctypes.byref(db), None), "apnn_conv_pair")
+    e3 = O.lowbits_pack(O.bn_quantize(acc3, None, thr3, None, xb), rows, cout, xb)
+    e1 = O.lowbits_pack(O.bn_quantize(acc1, None, thr1, None, xb), rows, cout, xb)
+    assert np.array_equal(G.to_host(o3, np.uint32).reshape(e3.shape), e3)
+    assert np.array_equal(G.to_host(o1, np.uint32).reshape(e1.shape), e1)
+    # descriptors that do not describe the same input / output grid are rejected
+    bad = desc(dW1, o1, 1, 0, dT1)
+    bad.stride = 1
+    assert A.lib().apnn_conv_pair(ctypes.byref(da), ctypes.byref(bad), None) == A.EINVAL
