@@ -345,59 +345,66 @@ struct EpiOperands {
 // rbase / cbase: first output row / column of this wave's tile.  Kernels whose waves tile the output
 // (KS == 1) quantize straight from the accumulators when the epilogue allows it (`direct`; codes of up
 // to DIRECT_BITS bits); split-K kernels and the remaining epilogues go through the slab.
-template <int KS, int DIRECT_BITS, int FA, int FB>
-__device__ __forceinline__ void epi_prefetch(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
+template <int KS, int FA, int FB>
+__device__ __forceinline__ void epi_load(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
   constexpr int NCOLS_E = FB * 32;
   constexpr int RES_REGS = FB;  // two planes x 32 rows x NCOLS/32 words over 64 lanes
   const int li = lane & 31;
+  if (p.epi == APNN_EPI_INT32) return;
+  if (eo.direct) {
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      const int gcol = cbase + y * 32 + li;
+      eo.thrT[y][0] = eo.thrT[y][1] = eo.thrT[y][2] = 0;
+      eo.flipm[y] = 0;
+      if (p.epi == APNN_EPI_BN && gcol < p.rowsB) {
+        eo.flipm[y] = (p.flip != nullptr && p.flip[gcol] != 0) ? -1 : 0;
+        if (p.out_bits <= 2) {
+          const int nt = (1 << p.out_bits) - 1;
+          const int32_t *t = p.thr + (long long)gcol * nt;
+          eo.thrT[y][0] = t[0];
+          eo.thrT[y][1] = nt > 1 ? t[1] : t[0];
+          eo.thrT[y][2] = nt > 2 ? t[2] : t[0];
+        }
+      }
+    }
+  } else if (KS > 1) {
+    load_tile_quant<NCOLS_E>(p, cbase, eo.q0, eo.q1);
+  }
+  if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (eo.direct || KS > 1)) {
+#pragma unroll
+    for (int x = 0; x < FA; ++x) {
+      if (KS == 1)
+        shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
+      else
+        shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
+    }
+    eo.res_prefetched = true;
+  }
+}
+
+// LAZY: only decide the output path now and fetch the operands in epi_finish (the largest tiles have no
+// registers to spare for values that are idle during the K loop).
+template <int KS, int DIRECT_BITS, bool LAZY, int FA, int FB>
+__device__ __forceinline__ void epi_prefetch(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
   eo.direct = KS == 1 && p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
               p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
   eo.q0 = ChannelQuant{};
   eo.q1 = ChannelQuant{};
   eo.res_prefetched = false;
-  if (p.epi != APNN_EPI_INT32) {
-    if (eo.direct) {
-#pragma unroll
-      for (int y = 0; y < FB; ++y) {
-        const int gcol = cbase + y * 32 + li;
-        eo.thrT[y][0] = eo.thrT[y][1] = eo.thrT[y][2] = 0;
-        eo.flipm[y] = 0;
-        if (p.epi == APNN_EPI_BN && gcol < p.rowsB) {
-          eo.flipm[y] = (p.flip != nullptr && p.flip[gcol] != 0) ? -1 : 0;
-          if (p.out_bits <= 2) {
-            const int nt = (1 << p.out_bits) - 1;
-            const int32_t *t = p.thr + (long long)gcol * nt;
-            eo.thrT[y][0] = t[0];
-            eo.thrT[y][1] = nt > 1 ? t[1] : t[0];
-            eo.thrT[y][2] = nt > 2 ? t[2] : t[0];
-          }
-        }
-      }
-    } else if (KS > 1) {
-      load_tile_quant<NCOLS_E>(p, cbase, eo.q0, eo.q1);
-    }
-    if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (eo.direct || KS > 1)) {
-#pragma unroll
-      for (int x = 0; x < FA; ++x) {
-        if (KS == 1)
-          shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
-        else
-          shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
-      }
-      eo.res_prefetched = true;
-    }
-  }
+  if (!LAZY) epi_load<KS>(p, rbase, cbase, lane, eo);
 }
 
 // Output stage of a work-group of four waves (WA x WB of them tile the output, KS = 4 / (WA*WB) split
 // K).  acc: this wave's FA x FB accumulator blocks; ssum: activation sums of the lane's row li of each
 // row block (convolution) or column li of each column block (GEMM entry points), complete in every
 // lane.  smem: the work-group's LDS, free for reuse after the barrier at the top.
-template <bool F4, int KS, bool CONV, int DIRECT_BITS, int FA, int FB, class AccT>
+template <bool F4, int KS, bool CONV, int DIRECT_BITS, bool LAZY, int FA, int FB, class AccT>
 __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB], const int (&ssum)[CONV ? FA : FB],
                                            uint32_t *smem, int wave, int lane, int a0, int b0, int wa, int wb,
                                            EpiOperands<FA, FB> &eo) {
   const int li = lane & 31, g = lane >> 5;
+  if (LAZY) epi_load<KS>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
   constexpr int RES_REGS = FB;
   const bool direct = eo.direct, res_prefetched = eo.res_prefetched;
   ChannelQuant &q0 = eo.q0, &q1 = eo.q1;
@@ -651,7 +658,8 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
 
   // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop
   EpiOperands<FA, FB> eo;
-  epi_prefetch<KS, (CONV ? PA : PB) >= 3 ? 4 : 2>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
+  constexpr bool EPI_LAZY = FA * FB >= 8;
+  epi_prefetch<KS, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
 
   // packed words of this lane's rows for one k-step
   uint32_t wA[FA][PA], wB[FB][PB];
@@ -799,7 +807,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     ssum[x] = t;
   }
 
-  epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
+  epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
 }
 
 constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
   for (int x = 0; x < FA; ++x) ssum[x] = 0;
 
   EpiOperands<FA, FB> eo;
-  epi_prefetch<1, DIRECT_BITS>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
+  epi_prefetch<1, DIRECT_BITS, false>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
 
   const bool pair_ok = (p.C32 & 1) == 0;  // 64-bit loads of a channel-word pair
   const int nchunks = (p.C32 + 1) >> 1;
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
       }
     }
   }
-  epi_finish<true, 1, true, DIRECT_BITS>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
+  epi_finish<true, 1, true, DIRECT_BITS, false>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
 }
 
 // LDS bytes of a launch: patch + filter block + pixel sums, at least the slab area of the output stage
