@@ -19,8 +19,11 @@ __device__ __forceinline__ int quantize_code(const KParams &p, int v, int gcol) 
   const int nt = (1 << p.out_bits) - 1;
   if (p.flip != nullptr && p.flip[gcol]) v = -v;
   const int32_t *t = p.thr + (long long)gcol * nt;
+  // the code is the number of thresholds <= v; the thresholds of a channel are sorted, so a binary
+  // search over the 2^bits - 1 of them finds it with one load per output bit
   int code = 0;
-  for (int k = 0; k < nt; ++k) code += (v >= t[k]) ? 1 : 0;
+  for (int h = (nt + 1) >> 1; h > 0; h >>= 1)
+    if (v >= t[code + h - 1]) code += h;
   return code;
 }
 
@@ -137,6 +140,37 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
   const bool res_global = p.resid_planes != nullptr && res_lds == nullptr;
   const bool res_local = p.resid_planes != nullptr && res_lds != nullptr;
 
+  // Codes of three or four bits: a lane meets one channel (two when the tile is 128 wide), so its 7 or
+  // 15 thresholds are fetched once into registers; the code is the number of thresholds <= v.
+  constexpr int NCH = NCOLS == 128 ? 2 : 1;
+  const bool wide = p.epi == APNN_EPI_BN && p.out_bits > 2 && p.out_bits <= 4;
+  const int nt = (1 << p.out_bits) - 1;
+  int tq[NCH][15];
+  int tflip[NCH] = {};  // 0 or -1
+  if (wide) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int gc = cbase + lane % NCOLS + 64 * c;
+      const int32_t *t = p.thr + (long long)(gc < p.rowsB ? gc : 0) * nt;
+#pragma unroll
+      for (int k = 0; k < 15; ++k) tq[c][k] = t[k < nt ? k : nt - 1];
+      tflip[c] = (p.flip != nullptr && gc < p.rowsB && p.flip[gc] != 0) ? -1 : 0;
+    }
+  }
+  auto quant = [&](const ChannelQuant &q, int c, int v, int gc) {
+    if (!wide) return quantize_with(p, q, v, gc);
+    const int fm = (NCH == 2 && c) ? tflip[NCH - 1] : tflip[0];
+    v = (v ^ fm) - fm;
+    int code = 0;
+#pragma unroll
+    for (int k = 0; k < 7; ++k) code += (v >= (NCH == 2 && c ? tq[NCH - 1][k] : tq[0][k])) ? 1 : 0;
+    if (nt > 7) {
+#pragma unroll
+      for (int k = 7; k < 15; ++k) code += (v >= (NCH == 2 && c ? tq[NCH - 1][k] : tq[0][k])) ? 1 : 0;
+    }
+    return code;
+  };
+
   for (int u0 = part; u0 < nunits; u0 += nparts * UB) {
     int v[UB], grow[UB], gcol[UB];
     bool ok[UB];
@@ -165,6 +199,7 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
       const int e = (u0 + j * nparts) * 64 + lane;
       const int orow = e / NCOLS, col = e % NCOLS;
       const ChannelQuant &q = (NCOLS == 128 && col >= 64) ? q1 : q0;
+      const int ch = (NCOLS == 128 && col >= 64) ? 1 : 0;
       int code = 0;
       if (ok[j]) {
         if (!pooled) {
@@ -179,15 +214,15 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
             t += rc * p.resid_scale;
           }
           if (p.save_acc != nullptr) p.save_acc[(long long)grow[j] * p.rowsB + gcol[j]] = t;
-          code = quantize_with(p, q, t, gcol[j]);
+          code = quant(q, ch, t, gcol[j]);
         } else {
           const int t0 = value(4 * orow, col), t1 = value(4 * orow + 1, col);
           const int t2 = value(4 * orow + 2, col), t3 = value(4 * orow + 3, col);
           if (p.pool == APNN_POOL_AVG2X2) {
-            code = quantize_with(p, q, (t0 + t1 + t2 + t3) / 4, gcol[j]);
+            code = quant(q, ch, (t0 + t1 + t2 + t3) / 4, gcol[j]);
           } else {
-            code = max(max(quantize_with(p, q, t0, gcol[j]), quantize_with(p, q, t1, gcol[j])),
-                       max(quantize_with(p, q, t2, gcol[j]), quantize_with(p, q, t3, gcol[j])));
+            code = max(max(quant(q, ch, t0, gcol[j]), quant(q, ch, t1, gcol[j])),
+                       max(quant(q, ch, t2, gcol[j]), quant(q, ch, t3, gcol[j])));
           }
         }
       }

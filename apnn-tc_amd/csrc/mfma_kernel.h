@@ -535,6 +535,27 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   const int a0 = (bid / tilesB) * TA;
   const int b0 = (bid % tilesB) * TB;
 
+  // output pixel (row of A) -> image index and the input coordinates of its filter tap (0, 0)
+  auto pixel_origin = [&](int pix, int &b, int &y0, int &x0) {
+    int oy, ox;
+    if (p.pool_order) {
+      const int win = pix >> 2, sub = pix & 3;
+      const int hw = p.Wo >> 1, hh = p.Ho >> 1;
+      const int px = win % hw, t = win / hw;
+      const int py = t % hh;
+      b = t / hh;
+      oy = 2 * py + (sub >> 1);
+      ox = 2 * px + (sub & 1);
+    } else {
+      ox = pix % p.Wo;
+      const int t = pix / p.Wo;
+      oy = t % p.Ho;
+      b = t / p.Ho;
+    }
+    y0 = oy * p.stride - p.pad;
+    x0 = ox * p.stride - p.pad;
+  };
+
   // ---- staging bookkeeping (same scheme as the VALU kernel) ----------------------------------
   int a_row[NIA], a_kq[NIA];
   int a_b[NIA], a_y0[NIA], a_x0[NIA];
@@ -546,26 +567,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     a_row[it] = u / KQ;
     const int grow = a0 + a_row[it];
     a_ok[it] = (u < UA) && (grow < p.rowsA);
-    if (CONV) {
-      int pix = grow, oy, ox, b;
-      if (p.pool_order) {
-        const int win = pix >> 2, sub = pix & 3;
-        const int hw = p.Wo >> 1, hh = p.Ho >> 1;
-        const int px = win % hw, t = win / hw;
-        const int py = t % hh;
-        b = t / hh;
-        oy = 2 * py + (sub >> 1);
-        ox = 2 * px + (sub & 1);
-      } else {
-        ox = pix % p.Wo;
-        const int t = pix / p.Wo;
-        oy = t % p.Ho;
-        b = t / p.Ho;
-      }
-      a_b[it] = b;
-      a_y0[it] = oy * p.stride - p.pad;
-      a_x0[it] = ox * p.stride - p.pad;
-    }
+    if (CONV) pixel_origin(grow, a_b[it], a_y0[it], a_x0[it]);
   }
   int b_row[NIB], b_kq[NIB];
   bool b_ok[NIB];
@@ -737,6 +739,73 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   constexpr int N_VALU = (F4 ? 7 : 8) * (FA * PA + FB * PB) + FS * PS;
   constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
 
+  // Split-K tiles with 128-bit loads: no wave shares an operand with another (each computes the whole
+  // tile over its own part of K), so the operands go from global memory straight into the registers the
+  // matrix core reads.  K is cut into groups of eight words; the lower lane half takes the first four
+  // words of a group and the upper half the last four, for both operands alike, which only permutes the
+  // terms of every dot product.  A wave requests GD groups at once (one memory latency per GD * KS
+  // groups of the work-group) and then runs four k-steps per group.
+  constexpr bool DIRECT_K = KS > 1 && VW == 4;
+  if constexpr (DIRECT_K) {
+    constexpr int GD_FIT = 48 / (4 * (PA + FB * PB));  // about 48 registers of operands in flight
+    constexpr int GD = GD_FIT < 1 ? 1 : GD_FIT;
+    const int ngroups = (p.KW + 7) >> 3;
+    const int growA = a0 + li;
+    const bool okA = growA < p.rowsA;
+    int ab = 0, ay0 = 0, ax0 = 0;
+    if (CONV) pixel_origin(growA, ab, ay0, ax0);
+    const uint32_t *rowA = p.A + (long long)growA * p.KW;  // GEMM entry points
+    const uint32_t *rowB[FB];
+    bool okB[FB];
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      okB[y] = b0 + y * 32 + li < p.rowsB;
+      rowB[y] = p.B + (long long)(b0 + y * 32 + li) * p.KW;
+    }
+    for (int gb = wave; gb < ngroups; gb += KS * GD) {
+      uint32_t ga[GD][PA][4], gbw[GD][FB][PB][4];
+#pragma unroll
+      for (int d = 0; d < GD; ++d) {
+        const int kw0 = (gb + d * KS) * 8 + 4 * g;
+        const bool in_k = kw0 < p.KW;
+        bool ok = okA && in_k;
+        const uint32_t *src;
+        if (CONV) {
+          const uint32_t tap = fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
+          const int cw = kw0 - (int)tap * p.C32;
+          const uint32_t r = fast_div(tap, (uint32_t)p.S, p.magicS);
+          const int s = (int)tap - (int)r * p.S;
+          const int iy = ay0 + (int)r, ix = ax0 + s;
+          ok = ok && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws;
+          src = p.A + ((((long long)ab * p.Hs + iy) * p.Ws + ix) * p.C32 + cw);
+        } else {
+          src = rowA + kw0;
+        }
+#pragma unroll
+        for (int pl = 0; pl < PA; ++pl) load_words<4>(src + pl * p.planeA, ok, ga[d][pl]);
+#pragma unroll
+        for (int y = 0; y < FB; ++y)
+#pragma unroll
+          for (int pl = 0; pl < PB; ++pl) load_words<4>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
+      }
+#pragma unroll
+      for (int d = 0; d < GD; ++d) {
+        if (gb + d * KS < ngroups) {  // same for the whole wave
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int pl = 0; pl < PA; ++pl) wA[0][pl] = ga[d][pl][i];
+#pragma unroll
+            for (int y = 0; y < FB; ++y)
+#pragma unroll
+              for (int pl = 0; pl < PB; ++pl) wB[y][pl] = gbw[d][y][pl][i];
+            expand_all(af, bf);
+            mfma_all();
+          }
+        }
+      }
+    }
+  } else {
   const int nchunks = (p.KW + KC - 1) / KC;
   fetch(0);
   stage(smem);
@@ -797,6 +866,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     mfma_all();
     if (more) advance();
   }
+  }
   int ssum[FS];
 #pragma unroll
   for (int x = 0; x < FS; ++x) {
@@ -812,7 +882,10 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
 
 constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
   const size_t ld = WA * WB == 1 ? 33 : (conv && FA * FB <= 2 && vw == 4) ? 17 : 9;  // KC + 1, see the kernel
-  const size_t stage = 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
+  // split-K tiles with 128-bit loads stage nothing (operands go from global memory to registers)
+  const size_t stage = WA * WB == 1 && vw == 4
+                           ? 0
+                           : 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
   const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
   return stage > slab ? stage : slab;
 }
