@@ -378,6 +378,12 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;
+  {
+    const int gw = p.pool_order ? Wo / 2 : Wo, gh = p.pool_order ? Ho / 2 : Ho;
+    p.magicGW = magic_of(gw);
+    p.magicGH = magic_of(gh);
+    p.geo_fast = ((unsigned long long)pixels + 1024) * (unsigned long long)(gw > gh ? gw : gh) < (1ull << 32);
+  }
   *vw_out = vw;
   return APNN_OK;
 }
@@ -405,8 +411,6 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
     if (pt >= 0) {
       p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
-      p.magicGW = magic_of(p.pool_order ? Wo / 2 : Wo);
-      p.magicGH = magic_of(p.pool_order ? Ho / 2 : Ho);
       p.magicPW = magic_of(p.PWs);
       p.magicPH = magic_of(p.PHs);
       return from_hip(pf(pt, p, stream));

@@ -36,6 +36,9 @@ struct KParams {
   // ceil(2^32/d) for the row grid (Wo, Ho; in pool order Wo/2, Ho/2) and the padded frame (PWs, PHs):
   // exact quotients for dividends below d + 1024
   uint32_t magicGW, magicGH, magicPW, magicPH;
+  // 1: every output row index times the larger of the row grid's sides stays below 2^32, so the
+  // matrix-core kernels may decode a row index into (image, y, x) with magicGW / magicGH
+  int geo_fast;
 
   // Paired launch (matrix-core convolution kernels only): work-groups pair_tiles .. 2*pair_tiles-1
   // compute a second convolution on the same input and output grid (same A, rows, columns, stride,

@@ -112,7 +112,9 @@ __device__ __forceinline__ int write_lane(int val, int old) {
 //   lds[0 .. FA*32)                          activation row sums (convolution, symmetric weights)
 //   lds[FA*32 .. FA*32 + FA*2*FB*32)         shortcut words, index ((x*2 + plane)*FB + y)*32 + row
 //   lds[FA*32 + FA*64*FB ...)                threshold table [k][FB*32] (TABLE only), filled here
-template <bool F4, int FA, int FB, bool CONV, bool TABLE, class AccT>
+// Q0, Q1: the register quads (rows 8q .. 8q+7 of a block) this call finishes; the split-K tiles give
+// each of their four waves one quad of the summed block.
+template <bool F4, int FA, int FB, bool CONV, bool TABLE, int Q0 = 0, int Q1 = 4, class AccT>
 __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA][FB],
                                                 const int (&ssum)[CONV ? FA : FB], uint32_t *lds, int rbase,
                                                 int cbase, int lane, const int (&T)[FB][3], const int (&fm)[FB],
@@ -152,7 +154,7 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
 #pragma unroll
       for (int k = 0; k < NPARK; ++k) park[y][k] = 0;
 
-    static_for<0, 4>([&](auto qc) {
+    static_for<Q0, Q1>([&](auto qc) {
       constexpr int q = decltype(qc)::value;
       int negc[4] = {0, 0, 0, 0};
       if (CONV) {
@@ -259,7 +261,8 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
     for (int k = 0; k < NPARK; ++k) {
       const int slot = 2 * k + (lane >> 5);
       const int plane = (TABLE && bn) ? nb - 1 - slot : slot;
-      if (plane >= 0 && plane < nb && row < rows_blk && grow < grow_end && gw0 < w32) {
+      const bool row_mine = (Q0 == 0 && Q1 == 4) || (pooled ? (row >= 2 * Q0 && row < 2 * Q1) : (row >= 8 * Q0 && row < 8 * Q1));
+      if (plane >= 0 && plane < nb && row < rows_blk && row_mine && grow < grow_end && gw0 < w32) {
         uint32_t *dst = out + plane * p.out_plane + (long long)grow * w32 + gw0;
         if (FB == 4 && (w32 & 3) == 0) {
           *reinterpret_cast<uint4 *>(dst) = make_uint4(park[0][k], park[FB > 1 ? 1 : 0][k], park[FB > 2 ? 2 : 0][k],
@@ -342,9 +345,9 @@ struct EpiOperands {
   uint32_t res_regs[FA][FB];
 };
 
-// rbase / cbase: first output row / column of this wave's tile.  Kernels whose waves tile the output
-// (KS == 1) quantize straight from the accumulators when the epilogue allows it (`direct`; codes of up
-// to DIRECT_BITS bits); split-K kernels and the remaining epilogues go through the slab.
+// rbase / cbase: first output row / column of this wave's tile.  Kernels quantize straight from the
+// accumulators when the epilogue allows it (`direct`; codes of up to DIRECT_BITS bits where the waves
+// tile the output, up to two bits in the split-K kernels); the remaining epilogues go through the slab.
 template <int KS, int FA, int FB>
 __device__ __forceinline__ void epi_load(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
   constexpr int NCOLS_E = FB * 32;
@@ -374,7 +377,7 @@ __device__ __forceinline__ void epi_load(const KParams &p, int rbase, int cbase,
   if (p.resid_planes != nullptr && p.resid_bits <= 2 && p.pool == APNN_POOL_NONE && (eo.direct || KS > 1)) {
 #pragma unroll
     for (int x = 0; x < FA; ++x) {
-      if (KS == 1)
+      if (eo.direct)
         shortcut_prefetch<NCOLS_E, RES_REGS, true>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
       else
         shortcut_prefetch<NCOLS_E, RES_REGS, false>(p, 32, rbase + x * 32, cbase, lane, 64, eo.res_regs[x]);
@@ -387,7 +390,7 @@ __device__ __forceinline__ void epi_load(const KParams &p, int rbase, int cbase,
 // registers to spare for values that are idle during the K loop).
 template <int KS, int DIRECT_BITS, bool LAZY, int FA, int FB>
 __device__ __forceinline__ void epi_prefetch(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
-  eo.direct = KS == 1 && p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
+  eo.direct = p.epi != APNN_EPI_INT32 && p.out_bits <= (KS == 1 ? DIRECT_BITS : 2) && p.resid == nullptr &&
               p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
   eo.q0 = ChannelQuant{};
   eo.q1 = ChannelQuant{};
@@ -421,6 +424,78 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
   constexpr int DIRECT_WORDS = FA * 32 + FA * 64 * FB + 15 * NCOLS;
   static_assert(DIRECT_WORDS <= SLAB_WORDS, "the register epilogue reuses the slab area");
   __syncthreads();  // every wave is done with the staging buffers
+  if constexpr (KS > 1) {
+    if (direct) {
+      // Split-K: the KS partial blocks meet in LDS in the accumulator's own register layout (16 bytes
+      // per lane and register quad), then wave q sums quad q of every column block -- rows 8q .. 8q+7 --
+      // and finishes it like a wave of the other kernels finishes its own accumulators.
+      using Acc4 = typename std::conditional<F4, float4, int4>::type;
+      constexpr int PART_WORDS = KS * FB * 4 * 64 * 4;
+      constexpr int SUM_WORDS = KS * FB * 32;
+      constexpr int AREA_WORDS = 32 + 64 * FB;
+      static_assert(PART_WORDS + SUM_WORDS + KS * AREA_WORDS <= KS * SLAB_WORDS, "fits the slab area");
+      Acc4 *part = reinterpret_cast<Acc4 *>(smem);
+      int *sums = reinterpret_cast<int *>(smem) + PART_WORDS;
+      uint32_t *area = smem + PART_WORDS + SUM_WORDS + wave * AREA_WORDS;
+      static_for<0, FB>([&](auto yc) {
+        constexpr int y = decltype(yc)::value;
+        static_for<0, 4>([&](auto qc) {
+          constexpr int q = decltype(qc)::value;
+          Acc4 v;
+          v.x = acc[0][y][4 * q];
+          v.y = acc[0][y][4 * q + 1];
+          v.z = acc[0][y][4 * q + 2];
+          v.w = acc[0][y][4 * q + 3];
+          part[((wave * FB + y) * 4 + q) * 64 + lane] = v;
+        });
+      });
+      if (g == 0) {
+#pragma unroll
+        for (int s = 0; s < (CONV ? 1 : FB); ++s) sums[(wave * FB + s) * 32 + li] = ssum[s];
+      }
+      if (res_prefetched) shortcut_publish<RES_REGS>(area + 32, lane, 64, res_regs[0]);
+      __syncthreads();
+      int stot[CONV ? FA : FB];
+#pragma unroll
+      for (int s = 0; s < (CONV ? 1 : FB); ++s) {
+        int t = 0;
+#pragma unroll
+        for (int w = 0; w < KS; ++w) t += sums[(w * FB + s) * 32 + li];
+        stot[s] = t;
+      }
+      if (CONV && g == 0) area[li] = (uint32_t)stot[0];
+      const int rb = a0, cb = b0;
+      auto finish_quad = [&](auto qc) {
+        constexpr int q = decltype(qc)::value;
+        AccT accr[1][FB];
+        static_for<0, FB>([&](auto yc) {
+          constexpr int y = decltype(yc)::value;
+          Acc4 t = part[(y * 4 + q) * 64 + lane];
+#pragma unroll
+          for (int w = 1; w < KS; ++w) {
+            const Acc4 u = part[((w * FB + y) * 4 + q) * 64 + lane];
+            t.x += u.x;
+            t.y += u.y;
+            t.z += u.z;
+            t.w += u.w;
+          }
+          accr[0][y][4 * q] = t.x;
+          accr[0][y][4 * q + 1] = t.y;
+          accr[0][y][4 * q + 2] = t.z;
+          accr[0][y][4 * q + 3] = t.w;
+        });
+        direct_epilogue<F4, 1, FB, CONV, false, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm, res_prefetched);
+      };
+      static_assert(KS == 4, "one register quad per wave");
+      switch (wave) {
+        case 0: finish_quad(std::integral_constant<int, 0>{}); break;
+        case 1: finish_quad(std::integral_constant<int, 1>{}); break;
+        case 2: finish_quad(std::integral_constant<int, 2>{}); break;
+        default: finish_quad(std::integral_constant<int, 3>{}); break;
+      }
+      return;
+    }
+  }
   if constexpr (KS == 1) {
     if (direct) {
       uint32_t *area = smem + wave * SLAB_WORDS;
@@ -538,7 +613,17 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   // output pixel (row of A) -> image index and the input coordinates of its filter tap (0, 0)
   auto pixel_origin = [&](int pix, int &b, int &y0, int &x0) {
     int oy, ox;
-    if (p.pool_order) {
+    if (p.geo_fast) {
+      // multiply-high by ceil(2^32 / d) is the exact quotient here (the host checked the range)
+      const int gw = p.pool_order ? p.Wo >> 1 : p.Wo, gh = p.pool_order ? p.Ho >> 1 : p.Ho;
+      const int cell = p.pool_order ? pix >> 2 : pix, sub = pix & 3;
+      const int t = (int)fast_div((uint32_t)cell, (uint32_t)gw, p.magicGW);
+      const int px = cell - t * gw;
+      b = (int)fast_div((uint32_t)t, (uint32_t)gh, p.magicGH);
+      const int py = t - b * gh;
+      oy = p.pool_order ? 2 * py + (sub >> 1) : py;
+      ox = p.pool_order ? 2 * px + (sub & 1) : px;
+    } else if (p.pool_order) {
       const int win = pix >> 2, sub = pix & 3;
       const int hw = p.Wo >> 1, hh = p.Ho >> 1;
       const int px = win % hw, t = win / hw;
@@ -747,7 +832,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   // groups of the work-group) and then runs four k-steps per group.
   constexpr bool DIRECT_K = KS > 1 && VW == 4;
   if constexpr (DIRECT_K) {
-    constexpr int GD_FIT = 48 / (4 * (PA + FB * PB));  // about 48 registers of operands in flight
+    constexpr int GD_FIT = (FB == 1 ? 60 : 48) / (4 * (PA + FB * PB));  // registers of operands in flight
     constexpr int GD = GD_FIT < 1 ? 1 : GD_FIT;
     const int ngroups = (p.KW + 7) >> 3;
     const int growA = a0 + li;
