@@ -109,7 +109,8 @@ __device__ __forceinline__ int write_lane(int val, int old) {
 // 4q..4q+3 of one lane, so pooling is register-local.
 //
 // Row-dependent terms come from LDS with 16-byte broadcast reads (four consecutive rows):
-//   lds[0 .. FA*32)                          activation row sums (convolution, symmetric weights)
+//   lds[0 .. FA*32)                          activation row sums times the weight range (convolution,
+//                                            symmetric weights; zero otherwise)
 //   lds[FA*32 .. FA*32 + FA*2*FB*32)         shortcut words, index ((x*2 + plane)*FB + y)*32 + row
 //   lds[FA*32 + FA*64*FB ...)                threshold table [k][FB*32] (TABLE only), filled here
 // Q0, Q1: the register quads (rows 8q .. 8q+7 of a block) this call finishes; the split-K tiles give
@@ -146,137 +147,156 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
 #pragma unroll
   for (int y = 0; y < FB; ++y) cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
 
-  static_for<0, FA>([&](auto xc) {
-    constexpr int x = decltype(xc)::value;
-    uint32_t park[FB][NPARK];
+  // The epilogue mode (thresholds or low bits, pooled or not) is the same for the whole launch: the
+  // value loop is instantiated once per mode and entered through one branch, so the per-value code
+  // carries no mode tests.
+  auto run = [&](auto bn_c, auto pooled_c) {
+    constexpr bool BN = decltype(bn_c)::value, POOLED = decltype(pooled_c)::value;
+    static_for<0, FA>([&](auto xc) {
+      constexpr int x = decltype(xc)::value;
+      uint32_t park[FB][NPARK];
 #pragma unroll
-    for (int y = 0; y < FB; ++y)
+      for (int y = 0; y < FB; ++y)
 #pragma unroll
-      for (int k = 0; k < NPARK; ++k) park[y][k] = 0;
+        for (int k = 0; k < NPARK; ++k) park[y][k] = 0;
 
-    static_for<Q0, Q1>([&](auto qc) {
-      constexpr int q = decltype(qc)::value;
-      int negc[4] = {0, 0, 0, 0};
-      if (CONV) {
-        const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
-        negc[0] = -wmax * rs.x;
-        negc[1] = -wmax * rs.y;
-        negc[2] = -wmax * rs.z;
-        negc[3] = -wmax * rs.w;
-      }
-      static_for<0, FB>([&](auto yc) {
-        constexpr int y = decltype(yc)::value;
-        uint32_t rw[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-        if (shortcut) {
-#pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            const uint4 w4 = *reinterpret_cast<const uint4 *>(res + ((x * 2 + b) * FB + y) * 32 + 8 * q + 4 * g);
-            rw[b][0] = w4.x;
-            rw[b][1] = w4.y;
-            rw[b][2] = w4.z;
-            rw[b][3] = w4.w;
-          }
+      static_for<Q0, Q1>([&](auto qc) {
+        constexpr int q = decltype(qc)::value;
+        int negc[4] = {0, 0, 0, 0};
+        if (CONV) {
+          // the row sums were multiplied by the weight range when they were written
+          const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
+          negc[0] = -rs.x;
+          negc[1] = -rs.y;
+          negc[2] = -rs.z;
+          negc[3] = -rs.w;
         }
-        int v[4];
-        static_for<0, 4>([&](auto jc) {
-          constexpr int j = decltype(jc)::value;
-          int t;
-          if constexpr (F4) {
-            t = __float2int_rn(acc[x][y][4 * q + j] * 4.0f);
-          } else {
-            t = acc[x][y][4 * q + j];
-          }
-          t = (t << sh) + (CONV ? negc[j] : cneg[y]);
-          if (shortcut) {
-            const int code = (int)(((rw[0][j] >> bitpos) & 1u) | (((rw[1][j] >> bitpos) & 1u) << 1));
-            t += code * p.resid_scale;
-          }
-          v[j] = t;
-        });
-        // one item: value (or code) -> one ballot per output bit, words parked at lanes rlo (lane
-        // half 0's row) and rhi (lane half 1's row)
-        auto emit = [&](int val, auto rlo_c, auto rhi_c) {
-          constexpr int rlo = decltype(rlo_c)::value, rhi = decltype(rhi_c)::value;
-          auto put = [&](auto slot_c, unsigned long long mask) {
-            constexpr int slot = decltype(slot_c)::value;
-            const int lo = (int)__brev((uint32_t)mask), hi = (int)__brev((uint32_t)(mask >> 32));
-            int reg = (int)park[y][slot >> 1];
-            reg = write_lane<rlo + 32 * (slot & 1)>(lo, reg);
-            reg = write_lane<rhi + 32 * (slot & 1)>(hi, reg);
-            park[y][slot >> 1] = (uint32_t)reg;
-          };
-          if (!bn) {
-            static_for<0, 2 * NPARK>([&](auto bc) {
-              constexpr int b = decltype(bc)::value;
-              if (b < nb) put(bc, __ballot((val >> b) & 1));
-            });
-          } else if constexpr (!TABLE) {
-            const bool hi1 = val >= T[y][1];
-            put(std::integral_constant<int, 1>{}, __ballot(hi1));
-            const int tsel = hi1 ? T[y][2] : T[y][0];
-            put(std::integral_constant<int, 0>{}, __ballot(val >= tsel));
-          } else {
-            int idx = (1 << (nb - 1)) - 1, h = 1 << (nb - 1);
-            static_for<0, 4>([&](auto lc) {
-              constexpr int lvl = decltype(lc)::value;
-              if (lvl < nb) {
-                h >>= 1;
-                const bool d = val >= tl[idx * NCOLS + y * 32 + li];
-                put(lc, __ballot(d));
-                idx += d ? h : -h;
-              }
-            });
-          }
-        };
-        auto flipped = [&](int t) { return (t ^ fm[y]) - fm[y]; };
-        if (!pooled) {
+        static_for<0, FB>([&](auto yc) {
+          constexpr int y = decltype(yc)::value;
+          int v[4];
           static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            emit(bn ? flipped(v[j]) : (v[j] & lowmask), std::integral_constant<int, 8 * q + j>{},
-                 std::integral_constant<int, 8 * q + 4 + j>{});
+            int t;
+            if constexpr (F4) {
+              t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+            } else {
+              t = acc[x][y][4 * q + j];
+            }
+            v[j] = (t << sh) + (CONV ? negc[j] : cneg[y]);
           });
-        } else {
-          int val;
-          if (p.pool == APNN_POOL_AVG2X2) {
-            const int a = (v[0] + v[1] + v[2] + v[3]) / 4;
-            val = bn ? flipped(a) : (a & lowmask);
-          } else if (bn) {
-            val = max(max(flipped(v[0]), flipped(v[1])), max(flipped(v[2]), flipped(v[3])));
-          } else {
-            val = max(max(v[0] & lowmask, v[1] & lowmask), max(v[2] & lowmask, v[3] & lowmask));
+          if (!POOLED && shortcut) {
+            uint32_t rw[2][4];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              const uint4 w4 = *reinterpret_cast<const uint4 *>(res + ((x * 2 + b) * FB + y) * 32 + 8 * q + 4 * g);
+              rw[b][0] = w4.x;
+              rw[b][1] = w4.y;
+              rw[b][2] = w4.z;
+              rw[b][3] = w4.w;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int code = (int)(((rw[0][j] >> bitpos) & 1u) | (((rw[1][j] >> bitpos) & 1u) << 1));
+              v[j] += code * p.resid_scale;
+            }
           }
-          emit(val, std::integral_constant<int, 2 * q>{}, std::integral_constant<int, 2 * q + 1>{});
-        }
+          // one item: value (or code) -> one ballot per output bit, words parked at lanes rlo (lane
+          // half 0's row) and rhi (lane half 1's row)
+          auto emit = [&](int val, auto rlo_c, auto rhi_c) {
+            constexpr int rlo = decltype(rlo_c)::value, rhi = decltype(rhi_c)::value;
+            auto put = [&](auto slot_c, unsigned long long mask) {
+              constexpr int slot = decltype(slot_c)::value;
+              // The bit reversal (channel c -> bit 31 - c%32) runs on the scalar unit, between the
+              // compare that produced the mask and the lane write that consumes it: a lane write (opaque
+              // assembly, which the compiler's hazard handling does not see) must not take its scalar
+              // source straight from a vector compare.
+              const int lo = (int)__brev((uint32_t)mask), hi = (int)__brev((uint32_t)(mask >> 32));
+              int reg = (int)park[y][slot >> 1];
+              reg = write_lane<rlo + 32 * (slot & 1)>(lo, reg);
+              reg = write_lane<rhi + 32 * (slot & 1)>(hi, reg);
+              park[y][slot >> 1] = (uint32_t)reg;
+            };
+            if constexpr (!BN) {
+              static_for<0, 2 * NPARK>([&](auto bc) {
+                constexpr int b = decltype(bc)::value;
+                if (b < nb) put(bc, __ballot((val >> b) & 1));
+              });
+            } else if constexpr (!TABLE) {
+              const bool hi1 = val >= T[y][1];
+              put(std::integral_constant<int, 1>{}, __ballot(hi1));
+              const int tsel = hi1 ? T[y][2] : T[y][0];
+              put(std::integral_constant<int, 0>{}, __ballot(val >= tsel));
+            } else {
+              int idx = (1 << (nb - 1)) - 1, h = 1 << (nb - 1);
+              static_for<0, 4>([&](auto lc) {
+                constexpr int lvl = decltype(lc)::value;
+                if (lvl < nb) {
+                  h >>= 1;
+                  const bool d = val >= tl[idx * NCOLS + y * 32 + li];
+                  put(lc, __ballot(d));
+                  idx += d ? h : -h;
+                }
+              });
+            }
+          };
+          auto flipped = [&](int t) { return (t ^ fm[y]) - fm[y]; };
+          if constexpr (!POOLED) {
+            static_for<0, 4>([&](auto jc) {
+              constexpr int j = decltype(jc)::value;
+              emit(BN ? flipped(v[j]) : (v[j] & lowmask), std::integral_constant<int, 8 * q + j>{},
+                   std::integral_constant<int, 8 * q + 4 + j>{});
+            });
+          } else {
+            int val;
+            if (p.pool == APNN_POOL_AVG2X2) {
+              const int a = (v[0] + v[1] + v[2] + v[3]) / 4;
+              val = BN ? flipped(a) : (a & lowmask);
+            } else if (BN) {
+              val = max(max(flipped(v[0]), flipped(v[1])), max(flipped(v[2]), flipped(v[3])));
+            } else {
+              val = max(max(v[0] & lowmask, v[1] & lowmask), max(v[2] & lowmask, v[3] & lowmask));
+            }
+            emit(val, std::integral_constant<int, 2 * q>{}, std::integral_constant<int, 2 * q + 1>{});
+          }
+        });
       });
-    });
 
-    // lane L holds, in park[y][k], the word of block row L%32 for slot 2k + L/32
-    const int row = lane & 31;
-    const int rows_blk = pooled ? 8 : 32;
-    const int grow = (pooled ? (rbase >> 2) + x * 8 : rbase + x * 32) + row;
-    const int grow_end = pooled ? (p.rowsA >> 2) : p.rowsA;
-    uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
-    const int gw0 = cbase >> 5;
+      // lane L holds, in park[y][k], the word of block row L%32 for slot 2k + L/32
+      const int row = lane & 31;
+      const int rows_blk = POOLED ? 8 : 32;
+      const int grow = (POOLED ? (rbase >> 2) + x * 8 : rbase + x * 32) + row;
+      const int grow_end = POOLED ? (p.rowsA >> 2) : p.rowsA;
+      uint32_t *out = reinterpret_cast<uint32_t *>(p.out);
+      const int gw0 = cbase >> 5;
 #pragma unroll
-    for (int k = 0; k < NPARK; ++k) {
-      const int slot = 2 * k + (lane >> 5);
-      const int plane = (TABLE && bn) ? nb - 1 - slot : slot;
-      const bool row_mine = (Q0 == 0 && Q1 == 4) || (pooled ? (row >= 2 * Q0 && row < 2 * Q1) : (row >= 8 * Q0 && row < 8 * Q1));
-      if (plane >= 0 && plane < nb && row < rows_blk && row_mine && grow < grow_end && gw0 < w32) {
-        uint32_t *dst = out + plane * p.out_plane + (long long)grow * w32 + gw0;
-        if (FB == 4 && (w32 & 3) == 0) {
-          *reinterpret_cast<uint4 *>(dst) = make_uint4(park[0][k], park[FB > 1 ? 1 : 0][k], park[FB > 2 ? 2 : 0][k],
-                                                       park[FB > 3 ? 3 : 0][k]);
-        } else if (FB == 2 && (w32 & 1) == 0) {
-          *reinterpret_cast<uint2 *>(dst) = make_uint2(park[0][k], park[FB > 1 ? 1 : 0][k]);
-        } else {
+      for (int k = 0; k < NPARK; ++k) {
+        const int slot = 2 * k + (lane >> 5);
+        const int plane = (TABLE && BN) ? nb - 1 - slot : slot;
+        const bool row_mine =
+            (Q0 == 0 && Q1 == 4) || (POOLED ? (row >= 2 * Q0 && row < 2 * Q1) : (row >= 8 * Q0 && row < 8 * Q1));
+        if (plane >= 0 && plane < nb && row < rows_blk && row_mine && grow < grow_end && gw0 < w32) {
+          uint32_t *dst = out + plane * p.out_plane + (long long)grow * w32 + gw0;
+          if (FB == 4 && (w32 & 3) == 0) {
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(park[0][k], park[FB > 1 ? 1 : 0][k], park[FB > 2 ? 2 : 0][k],
+                                                         park[FB > 3 ? 3 : 0][k]);
+          } else if (FB == 2 && (w32 & 1) == 0) {
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(park[0][k], park[FB > 1 ? 1 : 0][k]);
+          } else {
 #pragma unroll
-          for (int y = 0; y < FB; ++y)
-            if (gw0 + y < w32) dst[y] = park[y][k];
+            for (int y = 0; y < FB; ++y)
+              if (gw0 + y < w32) dst[y] = park[y][k];
+          }
         }
       }
-    }
-  });
+    });
+  };
+  using std::false_type;
+  using std::true_type;
+  if (bn) {
+    if (pooled) run(true_type{}, true_type{}); else run(true_type{}, false_type{});
+  } else {
+    if (pooled) run(false_type{}, true_type{}); else run(false_type{}, false_type{});
+  }
 }
 
 // Output stage of one wave for a 32-row slab of its tile, staged in LDS as slab[32][NCOLS + 1]
@@ -463,7 +483,7 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
         for (int w = 0; w < KS; ++w) t += sums[(w * FB + s) * 32 + li];
         stot[s] = t;
       }
-      if (CONV && g == 0) area[li] = (uint32_t)stot[0];
+      if (CONV && g == 0) area[li] = (uint32_t)((p.sym ? p.wmax : 0) * stot[0]);
       const int rb = a0, cb = b0;
       auto finish_quad = [&](auto qc) {
         constexpr int q = decltype(qc)::value;
@@ -501,7 +521,7 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
       uint32_t *area = smem + wave * SLAB_WORDS;
       if (CONV && g == 0) {
 #pragma unroll
-        for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)ssum[CONV ? x : 0];
+        for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)((p.sym ? p.wmax : 0) * ssum[CONV ? x : 0]);
       }
       if (res_prefetched) {
 #pragma unroll
@@ -557,6 +577,9 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
   });
 }
 
+
+// longest reduction (32-bit words) the one- and two-block convolution tiles load without staging
+constexpr int kDirectMaxKW = 40;
 
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
 __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
@@ -641,10 +664,18 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     x0 = ox * p.stride - p.pad;
   };
 
+  // how the operands reach the matrix core (see direct_loop below)
+  constexpr bool DIRECT_K = F4 && KS > 1 && VW == 4;
+  constexpr bool DIRECT_OPT = F4 && CONV && KS == 1 && FA == 1 && FB <= 2;
+  const bool direct_k = DIRECT_OPT && p.KW <= kDirectMaxKW;
+
   // ---- staging bookkeeping (same scheme as the VALU kernel) ----------------------------------
   int a_row[NIA], a_kq[NIA];
   int a_b[NIA], a_y0[NIA], a_x0[NIA];
   bool a_ok[NIA];
+  int b_row[NIB], b_kq[NIB];
+  bool b_ok[NIB];
+  if (!DIRECT_K && !direct_k) {
 #pragma unroll
   for (int it = 0; it < NIA; ++it) {
     const int u = tid + it * NT;
@@ -654,14 +685,13 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     a_ok[it] = (u < UA) && (grow < p.rowsA);
     if (CONV) pixel_origin(grow, a_b[it], a_y0[it], a_x0[it]);
   }
-  int b_row[NIB], b_kq[NIB];
-  bool b_ok[NIB];
 #pragma unroll
   for (int it = 0; it < NIB; ++it) {
     const int u = tid + it * NT;
     b_kq[it] = u % KQ;
     b_row[it] = u / KQ;
     b_ok[it] = (u < UB) && (b0 + b_row[it] < p.rowsB);
+  }
   }
 
   uint32_t ra_[NIA][PA][VW], rb_[NIB][PB][VW];
@@ -824,18 +854,23 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   constexpr int N_VALU = (F4 ? 7 : 8) * (FA * PA + FB * PB) + FS * PS;
   constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
 
-  // Split-K tiles with 128-bit loads: no wave shares an operand with another (each computes the whole
-  // tile over its own part of K), so the operands go from global memory straight into the registers the
-  // matrix core reads.  K is cut into groups of eight words; the lower lane half takes the first four
-  // words of a group and the upper half the last four, for both operands alike, which only permutes the
-  // terms of every dot product.  A wave requests GD groups at once (one memory latency per GD * KS
-  // groups of the work-group) and then runs four k-steps per group.
-  constexpr bool DIRECT_K = KS > 1 && VW == 4;
-  if constexpr (DIRECT_K) {
-    constexpr int GD_FIT = (FB == 1 ? 60 : 48) / (4 * (PA + FB * PB));  // registers of operands in flight
-    constexpr int GD = GD_FIT < 1 ? 1 : GD_FIT;
-    const int ngroups = (p.KW + 7) >> 3;
-    const int growA = a0 + li;
+  // Operands from global memory straight into the registers the matrix core reads -- no LDS staging, no
+  // barrier.  K is cut into groups of 2*VW words; the lower lane half takes the first VW words of a
+  // group and the upper half the last VW, for both operands alike, which only permutes the terms of
+  // every dot product.  A wave requests GD groups at once (one memory latency per batch) and then runs
+  // VW k-steps per group.  Used by
+  //   - the split-K tiles with 128-bit loads (always): no wave shares an operand with another there;
+  //   - the convolution tiles of one or two blocks per wave when the reduction is short (direct_k,
+  //     decided per launch): the waves of a work-group then load the rows they share once each, through
+  //     the L1 cache, which costs less than the staging pipeline's bookkeeping for a handful of k-steps.
+  auto direct_loop = [&]() {
+    constexpr int GW = 2 * VW;
+    constexpr int GD_FIT = (FB == 1 ? 60 : 48) / (VW * (PA + FB * PB));  // registers of operands in flight
+    constexpr int GD = GD_FIT < 1 ? 1 : (GD_FIT > 8 ? 8 : GD_FIT);
+    const int first = KS > 1 ? wave : 0;
+    constexpr int STEP = KS > 1 ? KS : 1;
+    const int ngroups = (p.KW + GW - 1) / GW;
+    const int growA = a0 + wa * FA * 32 + li;
     const bool okA = growA < p.rowsA;
     int ab = 0, ay0 = 0, ax0 = 0;
     if (CONV) pixel_origin(growA, ab, ay0, ax0);
@@ -844,14 +879,15 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     bool okB[FB];
 #pragma unroll
     for (int y = 0; y < FB; ++y) {
-      okB[y] = b0 + y * 32 + li < p.rowsB;
-      rowB[y] = p.B + (long long)(b0 + y * 32 + li) * p.KW;
+      const int grow = b0 + (wb * FB + y) * 32 + li;
+      okB[y] = grow < p.rowsB;
+      rowB[y] = p.B + (long long)grow * p.KW;
     }
-    for (int gb = wave; gb < ngroups; gb += KS * GD) {
-      uint32_t ga[GD][PA][4], gbw[GD][FB][PB][4];
+    for (int gb = first; gb < ngroups; gb += STEP * GD) {
+      uint32_t ga[GD][PA][VW], gbw[GD][FB][PB][VW];
 #pragma unroll
       for (int d = 0; d < GD; ++d) {
-        const int kw0 = (gb + d * KS) * 8 + 4 * g;
+        const int kw0 = (gb + d * STEP) * GW + VW * g;
         const bool in_k = kw0 < p.KW;
         bool ok = okA && in_k;
         const uint32_t *src;
@@ -867,17 +903,17 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
           src = rowA + kw0;
         }
 #pragma unroll
-        for (int pl = 0; pl < PA; ++pl) load_words<4>(src + pl * p.planeA, ok, ga[d][pl]);
+        for (int pl = 0; pl < PA; ++pl) load_words<VW>(src + pl * p.planeA, ok, ga[d][pl]);
 #pragma unroll
         for (int y = 0; y < FB; ++y)
 #pragma unroll
-          for (int pl = 0; pl < PB; ++pl) load_words<4>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
+          for (int pl = 0; pl < PB; ++pl) load_words<VW>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
       }
 #pragma unroll
       for (int d = 0; d < GD; ++d) {
-        if (gb + d * KS < ngroups) {  // same for the whole wave
+        if (gb + d * STEP < ngroups) {  // same for the whole wave
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
+          for (int i = 0; i < VW; ++i) {
 #pragma unroll
             for (int pl = 0; pl < PA; ++pl) wA[0][pl] = ga[d][pl][i];
 #pragma unroll
@@ -890,6 +926,11 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
         }
       }
     }
+  };
+  if constexpr (DIRECT_K) {
+    direct_loop();
+  } else if (direct_k) {
+    if constexpr (DIRECT_OPT) direct_loop();
   } else {
   const int nchunks = (p.KW + KC - 1) / KC;
   fetch(0);
