@@ -221,8 +221,9 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
   // cross-overs on ResNet18 / 16x16 benchmark shapes.
   if (conv) {
     const long long nb32 = ntiles(4);
-    if (KW >= 32 && nb32 <= 640) return 4;
-    if (KW >= 128 && nb32 <= 2560) return 5;
+    if (KW >= 32 && nb32 <= 256) return 4;   // at most one work-group per compute unit
+    if (KW >= 32 && nb32 <= 640) return 5;
+    if (KW >= 64 && nb32 <= 3200) return 5;
   }
   if (rowsB <= 64 && ntiles(3) >= cus) return 3;
   if (rowsB > 64) {

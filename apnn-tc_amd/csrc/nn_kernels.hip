@@ -343,8 +343,11 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
                                                            const int32_t *__restrict__ thr,
                                                            uint32_t *__restrict__ planes, int B, int H, int W, int C,
                                                            int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
-                                                           int bits, uint32_t xor_mask, int HPR, int NDW, int PWD) {
+                                                           int bits, uint32_t xor_mask, int HPR, int NDW, int PWD,
+                                                           uint32_t magic_gpr, uint32_t magic_ho) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // n / d by multiply-high with ceil(2^32 / d) where the launcher found it exact (magic != 0)
+  auto quot = [](uint32_t n, uint32_t d, uint32_t magic) { return magic != 0 ? __umulhi(n, magic) : n / d; };
   const int NH = R * HPR;
   const int nks = (NH + 1) / 2;
   const int KB = nks * 32, KPL = KB + 16;
@@ -436,9 +439,9 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   }
   uint32_t raw[NSLOT];
   auto request = [&](uint32_t grp, int base) {
-    const uint32_t trow = grp / (uint32_t)gpr;
+    const uint32_t trow = quot(grp, (uint32_t)gpr, magic_gpr);
     const int gx = (int)(grp - trow * (uint32_t)gpr);
-    const int b = (int)(trow / (uint32_t)Ho);
+    const int b = (int)quot(trow, (uint32_t)Ho, magic_ho);
     const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
     const int sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
     const uint8_t *img = X + (long long)b * H * rowbytes;
@@ -480,9 +483,9 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   uint32_t group = blockIdx.x * 4u + (uint32_t)wave;
   if (prefetch && group < ng) request(group, 0);
   for (; group < ng; group += gstep) {
-    const uint32_t trow = group / (uint32_t)gpr;
+    const uint32_t trow = quot(group, (uint32_t)gpr, magic_gpr);
     const int gx = (int)(group - trow * (uint32_t)gpr);
-    const int b = (int)(trow / (uint32_t)Ho);
+    const int b = (int)quot(trow, (uint32_t)Ho, magic_ho);
     const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
     const int ox0 = gx * 32;
     const int s0 = (ox0 * stride - pad) * C;
@@ -579,6 +582,8 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
 // ---- max-pool directly on bit-planes ----------------------------------------------------------------
 // in: [bits][B*H*W][cw] -> out: [bits][B*Ho*Wo][cw]; the maximum of two multi-bit codes is computed for
 // 32 channels at once with bitwise logic (compare from the top plane down).
+// NB: planes held in registers (2 for the usual one- and two-bit codes, else 8).
+template <int NB>
 __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
                                                           int B, int H, int W, int cw, int bits, int win, int stride,
                                                           int pad, int Ho, int Wo) {
@@ -604,9 +609,9 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__rest
       oy = (int)((row / Wo) % Ho);
       b = (int)(row / ((long long)Wo * Ho));
     }
-    uint32_t m[8];
+    uint32_t m[NB];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) m[p] = 0;
+    for (int p = 0; p < NB; ++p) m[p] = 0;
     for (int r = 0; r < win; ++r) {
       const int iy = oy * stride + r - pad;
       if (iy < 0 || iy >= H) continue;
@@ -614,21 +619,23 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__rest
         const int ix = ox * stride + sx - pad;
         if (ix < 0 || ix >= W) continue;
         const long long rin = ((long long)b * H + iy) * W + ix;
-        uint32_t v[8];
+        uint32_t v[NB];
 #pragma unroll
-        for (int p = 0; p < 8; ++p) v[p] = p < bits ? in[p * rows_in * cw + rin * cw + wi] : 0u;
+        for (int p = 0; p < NB; ++p) v[p] = p < bits ? in[p * rows_in * cw + rin * cw + wi] : 0u;
         uint32_t gt = 0, lt = 0;  // per channel: m > v decided / m < v decided
 #pragma unroll
-        for (int p = 7; p >= 0; --p) {
+        for (int p = NB - 1; p >= 0; --p) {
           const uint32_t diff = m[p] ^ v[p], open = ~(gt | lt);
           gt |= open & diff & m[p];
           lt |= open & diff & v[p];
         }
 #pragma unroll
-        for (int p = 0; p < 8; ++p) m[p] = (m[p] & ~lt) | (v[p] & lt);
+        for (int p = 0; p < NB; ++p) m[p] = (m[p] & ~lt) | (v[p] & lt);
       }
     }
-    for (int p = 0; p < bits; ++p) out[p * rows_out * cw + row * cw + wi] = m[p];
+#pragma unroll
+    for (int p = 0; p < NB; ++p)
+      if (p < bits) out[p * rows_out * cw + row * cw + wi] = m[p];
   }
 }
 
@@ -805,12 +812,18 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
       dim3 g2(grid.x > resident ? resident : grid.x, grid.y);
       const uint32_t xm = zero_point == 128 ? 0x80808080u : 0u;
       const uint8_t *Xu = reinterpret_cast<const uint8_t *>(X);
+      // multiply-high quotients for the pixel-group decode, where they are exact (n * d < 2^32)
+      const unsigned long long gpr = (unsigned long long)(Wo + 31) / 32, ngr = (unsigned long long)B * Ho * gpr;
+      auto magic = [&](unsigned long long d) {
+        return (d >= 2 && ngr * d < (1ull << 32)) ? (uint32_t)(((1ull << 32) + d - 1) / d) : 0u;
+      };
+      const uint32_t mg = magic(gpr), mh = magic((unsigned long long)Ho);
       if (wreg)
         hipLaunchKernelGGL(conv_i8_rows_kernel<7>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD);
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh);
       else
         hipLaunchKernelGGL(conv_i8_rows_kernel<0>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD);
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh);
       return hipGetLastError();
     }
   }
@@ -860,8 +873,12 @@ hipError_t launch_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, i
   const int Ho = (H + 2 * pad - win) / stride + 1, Wo = (W + 2 * pad - win) / stride + 1;
   long long blocks = ((long long)B * Ho * Wo * cw + 255) / 256;
   if (blocks > 262144) blocks = 262144;
-  hipLaunchKernelGGL(pool_planes_kernel, dim3((unsigned)blocks), dim3(256), 0, s, in, out, B, H, W, cw, bits, win,
-                     stride, pad, Ho, Wo);
+  if (bits <= 2)
+    hipLaunchKernelGGL(pool_planes_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, in, out, B, H, W, cw, bits, win,
+                       stride, pad, Ho, Wo);
+  else
+    hipLaunchKernelGGL(pool_planes_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, s, in, out, B, H, W, cw, bits, win,
+                       stride, pad, Ho, Wo);
   return hipGetLastError();
 }
 
