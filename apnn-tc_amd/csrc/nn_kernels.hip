@@ -344,10 +344,11 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
                                                            uint32_t *__restrict__ planes, int B, int H, int W, int C,
                                                            int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
                                                            int bits, uint32_t xor_mask, int HPR, int NDW, int PWD,
-                                                           uint32_t magic_gpr, uint32_t magic_ho) {
+                                                           uint32_t magic_gpr, uint32_t magic_ho, uint32_t magic_ndw,
+                                                           uint32_t magic_nh2, uint32_t magic_hpr, int wt_dwords) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   // n / d by multiply-high with ceil(2^32 / d) where the launcher found it exact (magic != 0)
-  auto quot = [](uint32_t n, uint32_t d, uint32_t magic) { return magic != 0 ? __umulhi(n, magic) : n / d; };
+  auto quot = [](uint32_t n, uint32_t d, uint32_t magic) { return magic != 0 ? __umulhi(n, magic) : (d == 1 ? n : n / d); };
   const int NH = R * HPR;
   const int nks = (NH + 1) / 2;
   const int KB = nks * 32, KPL = KB + 16;
@@ -364,27 +365,43 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   const int ntasks = 64 * nks * 2;
   for (int t0 = 0; t0 < ntasks; t0 += 4 * 256) {
     uint32_t w[4][4];
+    int dst_off[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int task = t0 + u * 256 + tid;
-      const int col = task / (nks * 2), hh = task - col * (nks * 2);
-      const int r = hh / HPR, hq = hh - r * HPR;
+      const int col = (int)quot((uint32_t)task, (uint32_t)(nks * 2), magic_nh2), hh = task - col * (nks * 2);
+      const int r = (int)quot((uint32_t)hh, (uint32_t)HPR, magic_hpr), hq = hh - r * HPR;
+      dst_off[u] = col * KPL + hh * 16;
       const int co = co0 + col;
       const int nvalid = (task < ntasks && co < COUT && r < R) ? min(max(SC - hq * 16, 0), 16) : 0;
       const int8_t *src = Wt + ((long long)co * R + r) * SC + hq * 16;
 #pragma unroll
       for (int q = 0; q < 4; ++q) w[u][q] = 0;
+      if (wt_dwords) {
+        // filter array readable as whole aligned dwords: five dword loads cover the 16 bytes at any
+        // byte offset, v_alignbyte shifts them into place, bytes past the row's end are masked off
+        const long long boff = src - Wt;
+        const uint32_t *wp = reinterpret_cast<const uint32_t *>(Wt) + (boff >> 2);
+        const uint32_t sh = (uint32_t)boff & 3u;
+        uint32_t d[5];
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (i < nvalid) w[u][i >> 2] |= (uint32_t)(uint8_t)src[i] << (8 * (i & 3));
+        for (int k = 0; k < 5; ++k) d[k] = (nvalid > 0 && 4 * k < (int)sh + nvalid) ? wp[k] : 0u;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int nb = min(max(nvalid - 4 * q, 0), 4);
+          const uint32_t mask = nb == 4 ? 0xffffffffu : ((1u << (8 * nb)) - 1u);
+          w[u][q] = __builtin_amdgcn_alignbyte(d[q + 1], d[q], sh) & mask;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (i < nvalid) w[u][i >> 2] |= (uint32_t)(uint8_t)src[i] << (8 * (i & 3));
+      }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int task = t0 + u * 256 + tid;
-      if (task < ntasks) {
-        const int col = task / (nks * 2), hh = task - col * (nks * 2);
-        *reinterpret_cast<uint4 *>(wl + col * KPL + hh * 16) = make_uint4(w[u][0], w[u][1], w[u][2], w[u][3]);
-      }
+      if (task < ntasks) *reinterpret_cast<uint4 *>(wl + dst_off[u]) = make_uint4(w[u][0], w[u][1], w[u][2], w[u][3]);
     }
   }
   __syncthreads();
@@ -434,7 +451,7 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
 #pragma unroll
   for (int j = 0; j < NSLOT; ++j) {
     const int idx = j * 64 + lane;
-    const int r = idx / NDW;
+    const int r = (int)quot((uint32_t)idx, (uint32_t)NDW, magic_ndw);
     rd[j] = idx < npatch ? ((r << 16) | (idx - r * NDW)) : -1;
   }
   uint32_t raw[NSLOT];
@@ -818,12 +835,17 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
         return (d >= 2 && ngr * d < (1ull << 32)) ? (uint32_t)(((1ull << 32) + d - 1) / d) : 0u;
       };
       const uint32_t mg = magic(gpr), mh = magic((unsigned long long)Ho);
+      // small dividends (patch slots below 512, filter tasks below 2^16): always exact
+      auto small_magic = [](int d) { return d >= 2 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
+      const uint32_t mn = small_magic(NDW), mt = small_magic(nks * 2), mp = small_magic(HPR);
+      // the filter array as aligned dwords: base 4-byte aligned and a whole number of dwords long
+      const int wt_dwords = (reinterpret_cast<uintptr_t>(Wt) & 3u) == 0 && ((long long)COUT * R * S * C) % 4 == 0;
       if (wreg)
         hipLaunchKernelGGL(conv_i8_rows_kernel<7>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh);
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh, mn, mt, mp, wt_dwords);
       else
         hipLaunchKernelGGL(conv_i8_rows_kernel<0>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh);
+                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh, mn, mt, mp, wt_dwords);
       return hipGetLastError();
     }
   }
