@@ -669,6 +669,70 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   constexpr bool DIRECT_OPT = F4 && CONV && KS == 1 && FA == 1 && FB <= 2;
   const bool direct_k = DIRECT_OPT && p.KW <= kDirectMaxKW;
 
+  // Operands from global memory straight into the registers the matrix core reads -- no LDS staging, no
+  // barrier.  K is cut into groups of 2*VW words; the lower lane half takes the first VW words of a
+  // group and the upper half the last VW, for both operands alike, which only permutes the terms of
+  // every dot product.  A wave requests GD groups at once (one memory latency per batch) and then runs
+  // VW k-steps per group.  Used by
+  //   - the split-K tiles with 128-bit loads (always): no wave shares an operand with another there;
+  //   - the convolution tiles of one or two blocks per wave when the reduction is short (direct_k,
+  //     decided per launch): the waves of a work-group then load the rows they share once each, through
+  //     the L1 cache, which costs less than the staging pipeline's bookkeeping for a handful of k-steps.
+  // The first batch is requested here, before thresholds, shortcut words and accumulators are set up,
+  // so that the rest of the prologue runs under its memory latency.
+  constexpr int GW = 2 * VW;
+  constexpr int GD_BUDGET = KS > 1 ? (FB == 1 ? 60 : 48) : (FB == 1 ? 40 : 32);  // registers of operands in flight
+  constexpr int GD_FIT = GD_BUDGET / (VW * (PA + FB * PB));
+  constexpr int GD = GD_FIT < 1 ? 1 : (GD_FIT > 8 ? 8 : GD_FIT);
+  constexpr int GSTEP = KS > 1 ? KS : 1;
+  const int gfirst = KS > 1 ? wave : 0;
+  const int ngroups = (p.KW + GW - 1) / GW;
+  uint32_t ga[GD][PA][VW], gbw[GD][FB][PB][VW];
+  bool okA = false;
+  int ab = 0, ay0 = 0, ax0 = 0;
+  const uint32_t *rowA = nullptr;
+  const uint32_t *rowB[FB];
+  bool okB[FB];
+  auto direct_issue = [&](int gb) {
+#pragma unroll
+    for (int d = 0; d < GD; ++d) {
+      const int kw0 = (gb + d * GSTEP) * GW + VW * g;
+      const bool in_k = kw0 < p.KW;
+      bool ok = okA && in_k;
+      const uint32_t *src;
+      if (CONV) {
+        const uint32_t tap = fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
+        const int cw = kw0 - (int)tap * p.C32;
+        const uint32_t r = fast_div(tap, (uint32_t)p.S, p.magicS);
+        const int s = (int)tap - (int)r * p.S;
+        const int iy = ay0 + (int)r, ix = ax0 + s;
+        ok = ok && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws;
+        src = p.A + ((((long long)ab * p.Hs + iy) * p.Ws + ix) * p.C32 + cw);
+      } else {
+        src = rowA + kw0;
+      }
+#pragma unroll
+      for (int pl = 0; pl < PA; ++pl) load_words<VW>(src + pl * p.planeA, ok, ga[d][pl]);
+#pragma unroll
+      for (int y = 0; y < FB; ++y)
+#pragma unroll
+        for (int pl = 0; pl < PB; ++pl) load_words<VW>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
+    }
+  };
+  if (DIRECT_K || direct_k) {
+    const int growA = a0 + wa * FA * 32 + li;
+    okA = growA < p.rowsA;
+    if (CONV) pixel_origin(growA, ab, ay0, ax0);
+    rowA = p.A + (long long)growA * p.KW;  // GEMM entry points
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      const int grow = b0 + (wb * FB + y) * 32 + li;
+      okB[y] = grow < p.rowsB;
+      rowB[y] = p.B + (long long)grow * p.KW;
+    }
+    direct_issue(gfirst);
+  }
+
   // ---- staging bookkeeping (same scheme as the VALU kernel) ----------------------------------
   int a_row[NIA], a_kq[NIA];
   int a_b[NIA], a_y0[NIA], a_x0[NIA];
@@ -854,64 +918,12 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   constexpr int N_VALU = (F4 ? 7 : 8) * (FA * PA + FB * PB) + FS * PS;
   constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
 
-  // Operands from global memory straight into the registers the matrix core reads -- no LDS staging, no
-  // barrier.  K is cut into groups of 2*VW words; the lower lane half takes the first VW words of a
-  // group and the upper half the last VW, for both operands alike, which only permutes the terms of
-  // every dot product.  A wave requests GD groups at once (one memory latency per batch) and then runs
-  // VW k-steps per group.  Used by
-  //   - the split-K tiles with 128-bit loads (always): no wave shares an operand with another there;
-  //   - the convolution tiles of one or two blocks per wave when the reduction is short (direct_k,
-  //     decided per launch): the waves of a work-group then load the rows they share once each, through
-  //     the L1 cache, which costs less than the staging pipeline's bookkeeping for a handful of k-steps.
   auto direct_loop = [&]() {
-    constexpr int GW = 2 * VW;
-    constexpr int GD_FIT = (FB == 1 ? 60 : 48) / (VW * (PA + FB * PB));  // registers of operands in flight
-    constexpr int GD = GD_FIT < 1 ? 1 : (GD_FIT > 8 ? 8 : GD_FIT);
-    const int first = KS > 1 ? wave : 0;
-    constexpr int STEP = KS > 1 ? KS : 1;
-    const int ngroups = (p.KW + GW - 1) / GW;
-    const int growA = a0 + wa * FA * 32 + li;
-    const bool okA = growA < p.rowsA;
-    int ab = 0, ay0 = 0, ax0 = 0;
-    if (CONV) pixel_origin(growA, ab, ay0, ax0);
-    const uint32_t *rowA = p.A + (long long)growA * p.KW;  // GEMM entry points
-    const uint32_t *rowB[FB];
-    bool okB[FB];
-#pragma unroll
-    for (int y = 0; y < FB; ++y) {
-      const int grow = b0 + (wb * FB + y) * 32 + li;
-      okB[y] = grow < p.rowsB;
-      rowB[y] = p.B + (long long)grow * p.KW;
-    }
-    for (int gb = first; gb < ngroups; gb += STEP * GD) {
-      uint32_t ga[GD][PA][VW], gbw[GD][FB][PB][VW];
+    for (int gb = gfirst; gb < ngroups; gb += GSTEP * GD) {
+      if (gb != gfirst) direct_issue(gb);  // the first batch is in flight since the prologue
 #pragma unroll
       for (int d = 0; d < GD; ++d) {
-        const int kw0 = (gb + d * STEP) * GW + VW * g;
-        const bool in_k = kw0 < p.KW;
-        bool ok = okA && in_k;
-        const uint32_t *src;
-        if (CONV) {
-          const uint32_t tap = fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
-          const int cw = kw0 - (int)tap * p.C32;
-          const uint32_t r = fast_div(tap, (uint32_t)p.S, p.magicS);
-          const int s = (int)tap - (int)r * p.S;
-          const int iy = ay0 + (int)r, ix = ax0 + s;
-          ok = ok && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws;
-          src = p.A + ((((long long)ab * p.Hs + iy) * p.Ws + ix) * p.C32 + cw);
-        } else {
-          src = rowA + kw0;
-        }
-#pragma unroll
-        for (int pl = 0; pl < PA; ++pl) load_words<VW>(src + pl * p.planeA, ok, ga[d][pl]);
-#pragma unroll
-        for (int y = 0; y < FB; ++y)
-#pragma unroll
-          for (int pl = 0; pl < PB; ++pl) load_words<VW>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
-      }
-#pragma unroll
-      for (int d = 0; d < GD; ++d) {
-        if (gb + d * STEP < ngroups) {  // same for the whole wave
+        if (gb + d * GSTEP < ngroups) {  // same for the whole wave
 #pragma unroll
           for (int i = 0; i < VW; ++i) {
 #pragma unroll
