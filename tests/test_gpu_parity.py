@@ -480,7 +480,7 @@ def test_pool_planes_wide_codes(G):
 @pytest.mark.parametrize("mode", ["bn", "lowbits"])
 @pytest.mark.parametrize("pool", [0, 1, 2])
 @pytest.mark.parametrize("xb,ob", [(2, 1), (2, 2), (2, 3), (3, 3), (4, 4), (4, 1), (3, 2), (2, 4)])
-@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (1, None), (4, 0), (4, 1), (4, 4)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (2, 5), (1, None), (4, 0), (4, 1), (4, 4)])
 def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
     rng = np.random.default_rng(4000 + 100 * xb + 10 * ob + pool + (tile or 0))
     batch, H, Wd, C, cout, wb = 2, 6, 10, 64, 96, 1
