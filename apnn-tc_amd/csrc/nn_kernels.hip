@@ -731,6 +731,48 @@ __global__ __launch_bounds__(256) void unpack_sum_kernel(const uint32_t *__restr
   }
 }
 
+// Pooled variant of the above for group >= 8 (global pooling of a feature map): one wave per (output
+// row, 32-channel word).  Lane j holds pixel j of the group (64 pixels per pass): one load per plane
+// and lane, all in flight together; the sum over the pixels of channel c's bit in plane b is the
+// population count of a wave-wide compare, accumulated in scalar registers.  Lane c stores channel c.
+__global__ __launch_bounds__(256) void pool_sum_kernel(const uint32_t *__restrict__ planes, int8_t *__restrict__ out,
+                                                       long long rows_out, int group, int C, int cpad, int bits,
+                                                       int shift) {
+  const int lane = threadIdx.x & 63;
+  const int cw = cpad >> 5;
+  const long long task = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (task >= rows_out * cw) return;  // the whole wave
+  const long long r = task / cw;
+  const int w = (int)(task - r * cw);
+  const long long rows_in = rows_out * group;
+  int cnt[32];
+#pragma unroll
+  for (int c = 0; c < 32; ++c) cnt[c] = 0;
+  for (int j0 = 0; j0 < group; j0 += 64) {
+    const int j = j0 + lane;
+    uint32_t wv[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+      wv[b] = (b < bits && j < group) ? planes[(long long)b * rows_in * cw + (r * group + j) * cw + w] : 0u;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      if (b < bits) {  // same for the whole wave
+        static_for_n<0, 32>([&](auto cc) {
+          constexpr int c = decltype(cc)::value;
+          cnt[c] += __popcll(__ballot((wv[b] >> (31 - c)) & 1u)) << b;
+        });
+      }
+    }
+  }
+  int mine = 0;
+  static_for_n<0, 32>([&](auto cc) {
+    constexpr int c = decltype(cc)::value;
+    if (lane == c) mine = cnt[c];
+  });
+  const int ch = w * 32 + lane;
+  if (lane < 32 && ch < C) out[r * C + ch] = (int8_t)min(127, mine >> shift);
+}
+
 // ---- int8 classifier: out[b][n] = scale[n] * sum_k X[b][k] * Wt[n][k] + bias[n] -----------------
 // One wave per (group of NN output features, group of four batch rows): lanes stride over K in dwords
 // (v_dot4_i32_i8 on four int8 pairs), every operand dword is used NN or four times, then wave64
@@ -917,6 +959,14 @@ hipError_t launch_pool_pack(const uint8_t *codes, uint32_t *planes, int B, int H
 
 hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int group, int C, int cpad,
                              int bits, int shift, hipStream_t s) {
+  if (group >= 8) {
+    const long long waves = rows_out * (cpad >> 5);
+    if ((waves + 3) / 4 <= 0x7fffffffLL) {
+      hipLaunchKernelGGL(pool_sum_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, planes, out, rows_out,
+                         group, C, cpad, bits, shift);
+      return hipGetLastError();
+    }
+  }
   int JP = 1;
   while (JP < 16 && JP * 2 <= group) JP *= 2;
   long long blocks = (rows_out * C * JP + 255) / 256;

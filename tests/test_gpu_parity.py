@@ -379,6 +379,21 @@ def test_unpack_sum_and_fc_i8(G):
     assert np.allclose(d_out.cpu().numpy().reshape(B, N), expect, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("B,HW,C,cpad,bits,shift", [(3, 150, 96, 96, 3, 2), (2, 64, 40, 64, 1, 0), (5, 9, 64, 64, 4, 0),
+                                                    (2, 7, 33, 64, 2, 0)])
+def test_unpack_sum_group_sizes(G, B, HW, C, cpad, bits, shift):
+    """Global pooling of packed codes: groups longer than a wave (several passes), a whole wave, short
+    groups (lane-split kernel), all code widths; sums saturate at 127."""
+    rng = np.random.default_rng(960 + HW)
+    codes = rng.integers(0, 1 << bits, size=(B * HW, C)).astype(np.uint32)
+    d_planes = G.to_dev(O.pack_bits(codes, B * HW, C, cpad, bits))
+    d_pool = torch.empty(B * C, dtype=torch.int8, device="cuda")
+    G.A.check(G.A.lib().apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_pool), B, HW, C, cpad, bits, shift, None), "pool")
+    torch.cuda.synchronize()
+    pooled = np.minimum(127, codes.reshape(B, HW, C).sum(1) >> shift).astype(np.int8)
+    assert np.array_equal(d_pool.cpu().numpy().reshape(B, C), pooled)
+
+
 @pytest.mark.parametrize("path,tile", CONV_TILES_PACKED + [(0, None)])
 def test_conv_packed_residual(G, path, tile):
     """Identity shortcut: the block input's packed codes are added, scaled, before the thresholds."""
