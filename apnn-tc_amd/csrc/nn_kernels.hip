@@ -629,6 +629,26 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__rest
     uint32_t m[NB];
 #pragma unroll
     for (int p = 0; p < NB; ++p) m[p] = 0;
+    if (NB == 2 && win == 3) {
+      // the usual 3x3 window on one- or two-bit codes: all eighteen loads are requested before the
+      // first compare (out-of-image taps read as code 0, the identity of the maximum)
+      uint32_t v[9][2];
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const int iy = oy * stride + t / 3 - pad, ix = ox * stride + t % 3 - pad;
+        const bool ok = iy >= 0 && iy < H && ix >= 0 && ix < W;
+        const long long rin = ((long long)b * H + iy) * W + ix;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) v[t][p] = (ok && p < bits) ? in[p * rows_in * cw + rin * cw + wi] : 0u;
+      }
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        // per channel: v > m  <=>  (v1 & ~m1) | (~(v1 ^ m1) & v0 & ~m0)
+        const uint32_t lt = (v[t][1] & ~m[1]) | (~(v[t][1] ^ m[1]) & v[t][0] & ~m[0]);
+        m[0] = (m[0] & ~lt) | (v[t][0] & lt);
+        m[1] = (m[1] & ~lt) | (v[t][1] & lt);
+      }
+    } else
     for (int r = 0; r < win; ++r) {
       const int iy = oy * stride + r - pad;
       if (iy < 0 || iy >= H) continue;
