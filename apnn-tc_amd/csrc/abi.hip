@@ -120,7 +120,9 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
 
 // what the register-only kernel (valu_direct_kernel.h) handles
 bool direct_kernel_serves(const KParams &p) {
-  if ((p.rowsB & 3) != 0 || (p.KW & 3) != 0) return false;
+  if ((p.rowsB & 3) != 0 || (p.KW & 3) != 0 || (p.rowsA + 3) / 4 > 65535) return false;
+  if ((unsigned long long)p.rowsA * p.KW * 4ull >= (1ull << 32) || (unsigned long long)p.rowsB * p.KW * 4ull >= (1ull << 32))
+    return false;  // the kernel addresses rows with 32-bit byte offsets
   if (p.epi == APNN_EPI_INT32) return true;
   return (p.rowsB & 31) == 0 && p.pool == APNN_POOL_NONE && p.resid == nullptr && p.save_acc == nullptr &&
          p.resid_planes == nullptr;

@@ -26,50 +26,53 @@
 
 namespace apnn {
 
-template <int PA, int PB, bool ACT_A>
+// QC: 128-bit word groups per lane, row and K step.  A lone wave on a SIMD issues one instruction every
+// four clocks, so the popcount work of a wave is on the launch's critical path: rows of at most 32 words
+// (eight groups, one per lane) run the QC = 1 instantiation, which does not carry a second, empty group.
+template <int PA, int PB, bool ACT_A, int QC>
 __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) {
-  constexpr int QC = 2;  // 128-bit word groups per lane, row and K step
   const int tid = threadIdx.x, lane = tid & 63;
   const int l = tid & 7;  // K slice
-  const int chunks_b = (p.rowsB + 31) >> 5;
-  const int ab = blockIdx.x / chunks_b, bc = blockIdx.x - ab * chunks_b;
+  const int ab = blockIdx.y, bc = blockIdx.x;  // four output rows x 32 columns per work-group
   const int a = ab * 4 + (tid >> 6);
   const int b = bc * 32 + ((tid & 63) >> 3) * 4;
   const bool live = a < p.rowsA && b < p.rowsB;
   const int nq = p.KW >> 2;  // 128-bit groups per row
-  const uint32_t *arow = p.A + (long long)a * p.KW;
-  const uint32_t *brow = p.B + (long long)b * p.KW;
+  // Loads are never predicated: a lane outside the problem (row, column or K slice past the end) reads
+  // the last valid row / group instead and its partial sums are dropped.  Addresses are a uniform
+  // plane base plus a 32-bit byte offset (the launcher checks that every row offset fits).
+  const uint32_t ac = (uint32_t)min(a, p.rowsA - 1), bcl = (uint32_t)(b < p.rowsB ? b : 0);
+  const uint32_t row_bytes = (uint32_t)p.KW * 4u;
+  const uint32_t offA = ac * row_bytes, offB = bcl * row_bytes;
 
   int acc[4] = {0, 0, 0, 0}, sx[4] = {0, 0, 0, 0};
   for (int q0 = 0; q0 < nq; q0 += 8 * QC) {
     uint4 wa[PA][QC], xb[4][PB][QC];
+    bool ok[QC];
 #pragma unroll
     for (int q = 0; q < QC; ++q) {
       const int qi = q0 + l + 8 * q;
-      const bool ok = live && qi < nq;
+      ok[q] = live && qi < nq;
+      const uint32_t koff = (uint32_t)min(qi, nq - 1) * 16u;
 #pragma unroll
-      for (int i = 0; i < PA; ++i) {
-        wa[i][q] = make_uint4(0, 0, 0, 0);
-        if (ok) wa[i][q] = *reinterpret_cast<const uint4 *>(arow + i * p.planeA + 4 * qi);
-      }
+      for (int i = 0; i < PA; ++i)
+        wa[i][q] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(p.A + i * p.planeA) + (offA + koff));
 #pragma unroll
       for (int o = 0; o < 4; ++o)
 #pragma unroll
-        for (int j = 0; j < PB; ++j) {
-          xb[o][j][q] = make_uint4(0, 0, 0, 0);
-          if (ok) xb[o][j][q] = *reinterpret_cast<const uint4 *>(brow + j * p.planeB + (long long)o * p.KW + 4 * qi);
-        }
+        for (int j = 0; j < PB; ++j)
+          xb[o][j][q] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(p.B + j * p.planeB) +
+                                                         (offB + (uint32_t)o * row_bytes + koff));
     }
 #pragma unroll
     for (int q = 0; q < QC; ++q) {
+      int tacc[4] = {0, 0, 0, 0}, tsx[4] = {0, 0, 0, 0};
       if (ACT_A) {
-        int s = 0;
 #pragma unroll
         for (int i = 0; i < PA; ++i) {
           const uint4 w = wa[i][q];
-          s += (__popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w)) << i;
+          tsx[0] += (__popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w)) << i;
         }
-        sx[0] += s;
       }
 #pragma unroll
       for (int o = 0; o < 4; ++o) {
@@ -79,20 +82,30 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
 #pragma unroll
           for (int i = 0; i < PA; ++i) {
             const uint4 w = wa[i][q];
-            acc[o] += (__popc(w.x & x.x) + __popc(w.y & x.y) + __popc(w.z & x.z) + __popc(w.w & x.w)) << (i + j);
+            tacc[o] += (__popc(w.x & x.x) + __popc(w.y & x.y) + __popc(w.z & x.z) + __popc(w.w & x.w)) << (i + j);
           }
-          if (!ACT_A) sx[o] += (__popc(x.x) + __popc(x.y) + __popc(x.z) + __popc(x.w)) << j;
+          if (!ACT_A) tsx[o] += (__popc(x.x) + __popc(x.y) + __popc(x.z) + __popc(x.w)) << j;
         }
+      }
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        acc[o] += ok[q] ? tacc[o] : 0;
+        sx[o] += ok[q] ? tsx[o] : 0;
       }
     }
   }
   int v[4];
 #pragma unroll
   for (int o = 0; o < 4; ++o) v[o] = p.sym ? 2 * acc[o] - p.wmax * sx[ACT_A ? 0 : o] : acc[o];
+  // butterfly over the eight lanes of a group with data-parallel-primitive adds: lane ^ 1 and lane ^ 2
+  // inside a quad, then the mirror image within eight lanes (every lane of a quad already holds the
+  // quad's sum, so lane 7 - i delivers the other quad's)
 #pragma unroll
-  for (int off = 1; off < 8; off <<= 1)
-#pragma unroll
-    for (int o = 0; o < 4; ++o) v[o] += __shfl_xor(v[o], off, 64);
+  for (int o = 0; o < 4; ++o) {
+    v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
+    v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+    v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x141, 0xf, 0xf, true);  // row_half_mirror
+  }
   const int mine = l == 0 ? v[0] : l == 1 ? v[1] : l == 2 ? v[2] : v[3];  // output column b + l for l < 4
 
   if (p.epi == APNN_EPI_INT32) {
@@ -130,8 +143,15 @@ inline hipError_t launch_valu_direct(const KParams &p, hipStream_t stream) {
       ((p.rowsB & 31) != 0 || p.pool != APNN_POOL_NONE || p.resid != nullptr || p.save_acc != nullptr ||
        p.resid_planes != nullptr))
     return hipErrorNotSupported;
-  const unsigned blocks = (unsigned)(((p.rowsA + 3) / 4) * ((p.rowsB + 31) / 32));
-  hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A>), dim3(blocks), dim3(256), 0, stream, p);
+  if ((p.rowsA + 3) / 4 > 65535) return hipErrorNotSupported;  // grid.y
+  // 32-bit byte offsets inside a plane
+  if ((unsigned long long)p.rowsA * p.KW * 4ull >= (1ull << 32) || (unsigned long long)p.rowsB * p.KW * 4ull >= (1ull << 32))
+    return hipErrorNotSupported;
+  const dim3 grid((unsigned)((p.rowsB + 31) / 32), (unsigned)((p.rowsA + 3) / 4));
+  if (p.KW <= 32)
+    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 1>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 2>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 
