@@ -26,6 +26,16 @@
 
 namespace apnn {
 
+// popc(x) + acc in one instruction (the compiler otherwise counts into fresh registers and adds the
+// counts in a tree, one more instruction per three words)
+__device__ __forceinline__ int popc_acc(uint32_t x, int acc) {
+  int r;
+  asm("v_bcnt_u32_b32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(acc));
+  return r;
+}
+__device__ __forceinline__ int popc4_acc(const uint4 &x, int acc) {
+  return popc_acc(x.w, popc_acc(x.z, popc_acc(x.y, popc_acc(x.x, acc))));
+}
 // QC: 128-bit word groups per lane, row and K step.  A lone wave on a SIMD issues one instruction every
 // four clocks, so the popcount work of a wave is on the launch's critical path: rows of at most 32 words
 // (eight groups, one per lane) run the QC = 1 instantiation, which does not carry a second, empty group.
@@ -45,6 +55,12 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   const uint32_t row_bytes = (uint32_t)p.KW * 4u;
   const uint32_t offA = ac * row_bytes, offB = bcl * row_bytes;
 
+  const char *baseA[PA], *baseB[PB];
+#pragma unroll
+  for (int i = 0; i < PA; ++i) baseA[i] = reinterpret_cast<const char *>(p.A + i * p.planeA);
+#pragma unroll
+  for (int j = 0; j < PB; ++j) baseB[j] = reinterpret_cast<const char *>(p.B + j * p.planeB);
+
   int acc[4] = {0, 0, 0, 0}, sx[4] = {0, 0, 0, 0};
   for (int q0 = 0; q0 < nq; q0 += 8 * QC) {
     uint4 wa[PA][QC], xb[4][PB][QC];
@@ -56,13 +72,12 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
       const uint32_t koff = (uint32_t)min(qi, nq - 1) * 16u;
 #pragma unroll
       for (int i = 0; i < PA; ++i)
-        wa[i][q] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(p.A + i * p.planeA) + (offA + koff));
+        wa[i][q] = *reinterpret_cast<const uint4 *>(baseA[i] + (offA + koff));
 #pragma unroll
       for (int o = 0; o < 4; ++o)
 #pragma unroll
         for (int j = 0; j < PB; ++j)
-          xb[o][j][q] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(p.B + j * p.planeB) +
-                                                         (offB + (uint32_t)o * row_bytes + koff));
+          xb[o][j][q] = *reinterpret_cast<const uint4 *>(baseB[j] + (offB + (uint32_t)o * row_bytes + koff));
     }
 #pragma unroll
     for (int q = 0; q < QC; ++q) {
@@ -70,8 +85,7 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
       if (ACT_A) {
 #pragma unroll
         for (int i = 0; i < PA; ++i) {
-          const uint4 w = wa[i][q];
-          tsx[0] += (__popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w)) << i;
+          tsx[0] += popc4_acc(wa[i][q], 0) << i;
         }
       }
 #pragma unroll
@@ -82,9 +96,12 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
 #pragma unroll
           for (int i = 0; i < PA; ++i) {
             const uint4 w = wa[i][q];
-            tacc[o] += (__popc(w.x & x.x) + __popc(w.y & x.y) + __popc(w.z & x.z) + __popc(w.w & x.w)) << (i + j);
+            const uint4 m = make_uint4(w.x & x.x, w.y & x.y, w.z & x.z, w.w & x.w);
+            if (i + j == 0) tacc[o] = popc4_acc(m, tacc[o]); else tacc[o] += popc4_acc(m, 0) << (i + j);
           }
-          if (!ACT_A) tsx[o] += (__popc(x.x) + __popc(x.y) + __popc(x.z) + __popc(x.w)) << j;
+          if (!ACT_A) {
+            if (j == 0) tsx[o] = popc4_acc(x, tsx[o]); else tsx[o] += popc4_acc(x, 0) << j;
+          }
         }
       }
 #pragma unroll
