@@ -39,13 +39,18 @@ __device__ __forceinline__ int popc4_acc(const uint4 &x, int acc) {
 // QC: 128-bit word groups per lane, row and K step.  A lone wave on a SIMD issues one instruction every
 // four clocks, so the popcount work of a wave is on the launch's critical path: rows of at most 32 words
 // (eight groups, one per lane) run the QC = 1 instantiation, which does not carry a second, empty group.
-template <int PA, int PB, bool ACT_A, int QC>
+// LPG: lanes that share four outputs and split K (8, or 4: a wave then owns 64 columns and the launch has
+// half as many waves, each with the same fixed cost and twice the popcount work -- taken when eight
+// lanes per group would put more than one wave on a SIMD).
+template <int PA, int PB, bool ACT_A, int QC, int LPG>
 __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) {
+  static_assert(LPG == 8 || LPG == 4, "lanes per output group");
+  constexpr int CPW = 64 / LPG * 4;  // columns per wave
   const int tid = threadIdx.x, lane = tid & 63;
-  const int l = tid & 7;  // K slice
-  const int ab = blockIdx.y, bc = blockIdx.x;  // four output rows x 32 columns per work-group
+  const int l = tid & (LPG - 1);  // K slice
+  const int ab = blockIdx.y, bc = blockIdx.x;  // four output rows x CPW columns per work-group
   const int a = ab * 4 + (tid >> 6);
-  const int b = bc * 32 + ((tid & 63) >> 3) * 4;
+  const int b = bc * CPW + ((tid & 63) / LPG) * 4;
   const bool live = a < p.rowsA && b < p.rowsB;
   const int nq = p.KW >> 2;  // 128-bit groups per row
   // Loads are never predicated: a lane outside the problem (row, column or K slice past the end) reads
@@ -62,12 +67,12 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   for (int j = 0; j < PB; ++j) baseB[j] = reinterpret_cast<const char *>(p.B + j * p.planeB);
 
   int acc[4] = {0, 0, 0, 0}, sx[4] = {0, 0, 0, 0};
-  for (int q0 = 0; q0 < nq; q0 += 8 * QC) {
+  for (int q0 = 0; q0 < nq; q0 += LPG * QC) {
     uint4 wa[PA][QC], xb[4][PB][QC];
     bool ok[QC];
 #pragma unroll
     for (int q = 0; q < QC; ++q) {
-      const int qi = q0 + l + 8 * q;
+      const int qi = q0 + l + LPG * q;
       ok[q] = live && qi < nq;
       const uint32_t koff = (uint32_t)min(qi, nq - 1) * 16u;
 #pragma unroll
@@ -121,12 +126,38 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   for (int o = 0; o < 4; ++o) {
     v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
     v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
-    v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x141, 0xf, 0xf, true);  // row_half_mirror
+    if (LPG == 8) v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x141, 0xf, 0xf, true);  // row_half_mirror
   }
-  const int mine = l == 0 ? v[0] : l == 1 ? v[1] : l == 2 ? v[2] : v[3];  // output column b + l for l < 4
+  const int l4 = l & 3;
+  const int mine = l4 == 0 ? v[0] : l4 == 1 ? v[1] : l4 == 2 ? v[2] : v[3];  // output column b + l for l < 4
 
   if (p.epi == APNN_EPI_INT32) {
     if (live && l < 4) reinterpret_cast<int *>(p.out)[(long long)a * p.rowsB + b + l] = mine;
+    return;
+  }
+  if constexpr (LPG == 4) {
+    // packed output, four lanes per group: lane L holds column bc*64 + L, so one ballot per output
+    // bit-plane is two finished words
+    int val = mine;
+    const int col = bc * 64 + lane;
+    const bool col_ok = col < p.rowsB;
+    int code = 0;
+    if (p.epi == APNN_EPI_LOWBITS) {
+      code = val & ((1 << p.out_bits) - 1);
+    } else if (col_ok) {
+      const int nt = (1 << p.out_bits) - 1;
+      if (p.flip != nullptr && p.flip[col]) val = -val;
+      const int32_t *t = p.thr + (long long)col * nt;
+      for (int k = 0; k < nt; ++k) code += (val >= t[k]) ? 1 : 0;
+    }
+    const int w32 = p.rowsB >> 5;
+    for (int bit = 0; bit < p.out_bits; ++bit) {
+      const unsigned long long mask = __ballot(col_ok && ((code >> bit) & 1));
+      const int wi = 2 * bc + (lane >> 5);
+      if ((lane & 31) == 0 && a < p.rowsA && wi < w32)
+        reinterpret_cast<uint32_t *>(p.out)[bit * p.out_plane + (long long)a * w32 + wi] =
+            __brev((uint32_t)(lane == 0 ? mask : mask >> 32));
+    }
     return;
   }
   // packed output: bring the 32 outputs of the wave to lanes 0..31 in column order, quantize each in
@@ -164,11 +195,26 @@ inline hipError_t launch_valu_direct(const KParams &p, hipStream_t stream) {
   // 32-bit byte offsets inside a plane
   if ((unsigned long long)p.rowsA * p.KW * 4ull >= (1ull << 32) || (unsigned long long)p.rowsB * p.KW * 4ull >= (1ull << 32))
     return hipErrorNotSupported;
-  const dim3 grid((unsigned)((p.rowsB + 31) / 32), (unsigned)((p.rowsA + 3) / 4));
-  if (p.KW <= 32)
-    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 1>), grid, dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 2>), grid, dim3(256), 0, stream, p);
+  static int cus = 0;  // compute units of the device (one device per process here)
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  const unsigned rows4 = (unsigned)((p.rowsA + 3) / 4);
+  const dim3 grid8((unsigned)((p.rowsB + 31) / 32), rows4), grid4((unsigned)((p.rowsB + 63) / 64), rows4);
+  if (grid8.x * rows4 > (unsigned)cus && p.KW <= 16) {
+    // rows of at most four word groups, more work-groups than compute units with eight lanes per group:
+    // four lanes per group, one word group each (with two word groups per lane, K = 1024, the longer
+    // popcount chain of a wave measured slower than two waves per SIMD: 2.55 vs 2.36 us)
+    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 1, 4>), grid4, dim3(256), 0, stream, p);
+  } else if (p.KW <= 32) {
+    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 1, 8>), grid8, dim3(256), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((apnn_valu_direct_kernel<PA, PB, ACT_A, 2, 8>), grid8, dim3(256), 0, stream, p);
+  }
   return hipGetLastError();
 }
 

@@ -639,9 +639,10 @@ def test_quantize_pack(G, bits, rows, C, cpad):
 
 @pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("wb,xb", COMBOS)
-@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (50, 36, 128), (1, 4, 2048), (64, 128, 1536), (7, 260, 640), (8, 64, 9216)])
+@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (50, 36, 128), (1, 4, 2048), (64, 128, 1536), (7, 260, 640), (8, 64, 9216),
+                                   (61, 1060, 512), (30, 2052, 768)])
 def test_gemm_register_only_kernel(G, M, N, K, wb, xb, sym):
-    """The latency-oriented GEMM kernel (eight lanes split K for four outputs), pinned as VALU tile 4."""
+    """The latency-oriented GEMM kernel (eight or four lanes split K for four outputs), pinned as VALU tile 4."""
     rng = np.random.default_rng(7000 + M + N + K + 10 * wb + xb + sym)
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
@@ -666,7 +667,7 @@ def test_gemm_register_only_kernel_limits(G):
 
 @pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("wb,xb,ob", [(1, 2, 2), (1, 4, 4), (2, 2, 1), (1, 3, 3)])
-@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (9, 96, 4096), (5, 32, 384)])
+@pytest.mark.parametrize("M,N,K", [(64, 1024, 1024), (9, 96, 4096), (5, 32, 384), (61, 1056, 512), (33, 2080, 896)])
 def test_gemm_register_only_kernel_packed(G, M, N, K, wb, xb, ob, sym):
     rng = np.random.default_rng(7200 + M + N + 10 * wb + xb + sym)
     W = O.random_planes(rng, wb, M, K // 32)
