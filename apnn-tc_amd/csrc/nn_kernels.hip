@@ -816,6 +816,8 @@ __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0;
   if (vec_ok) {
+    // four independent iterations in flight: a long K would otherwise be one memory round trip per step
+#pragma unroll 4
     for (int k4 = lane; k4 < (K >> 2); k4 += 64) {
       int wv[NN], xv[4];
 #pragma unroll
