@@ -117,8 +117,11 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
     }
   }
   int v[4];
+  // symmetric weights: 2 * raw - wmax * (activation sum), written without a branch (shift 0 and weight
+  // range 0 for the plain result)
+  const int sym_sh = p.sym ? 1 : 0, sym_w = p.sym ? p.wmax : 0;
 #pragma unroll
-  for (int o = 0; o < 4; ++o) v[o] = p.sym ? 2 * acc[o] - p.wmax * sx[ACT_A ? 0 : o] : acc[o];
+  for (int o = 0; o < 4; ++o) v[o] = (acc[o] << sym_sh) - sym_w * sx[ACT_A ? 0 : o];
   // butterfly over the eight lanes of a group with data-parallel-primitive adds: lane ^ 1 and lane ^ 2
   // inside a quad, then the mirror image within eight lanes (every lane of a quad already holds the
   // quad's sum, so lane 7 - i delivers the other quad's)
@@ -129,7 +132,9 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
     if (LPG == 8) v[o] += __builtin_amdgcn_update_dpp(0, v[o], 0x141, 0xf, 0xf, true);  // row_half_mirror
   }
   const int l4 = l & 3;
-  const int mine = l4 == 0 ? v[0] : l4 == 1 ? v[1] : l4 == 2 ? v[2] : v[3];  // output column b + l for l < 4
+  // output column b + l for l < 4 (two levels of selects, no branches)
+  const int m01 = (l4 & 1) ? v[1] : v[0], m23 = (l4 & 1) ? v[3] : v[2];
+  const int mine = (l4 & 2) ? m23 : m01;
 
   if (p.epi == APNN_EPI_INT32) {
     if (live && l < 4) reinterpret_cast<int *>(p.out)[(long long)a * p.rowsB + b + l] = mine;
