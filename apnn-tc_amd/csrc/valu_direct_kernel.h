@@ -65,6 +65,13 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   for (int i = 0; i < PA; ++i) baseA[i] = reinterpret_cast<const char *>(p.A + i * p.planeA);
 #pragma unroll
   for (int j = 0; j < PB; ++j) baseB[j] = reinterpret_cast<const char *>(p.B + j * p.planeB);
+  // Everything the kernel reads from its argument block is requested here, in one round of scalar
+  // loads, instead of a second round before the operand loads and a third after the K loop.
+  const int sym_sh = p.sym ? 1 : 0, sym_w = p.sym ? p.wmax : 0;
+  const int epi = p.epi;
+  int *out_i32 = reinterpret_cast<int *>(p.out);
+  asm volatile("" ::"s"(baseA[0]), "s"(baseB[0]), "s"(baseA[PA - 1]), "s"(baseB[PB - 1]), "s"(out_i32), "s"(sym_sh), "s"(sym_w),
+               "s"(epi));
 
   int acc[4] = {0, 0, 0, 0}, sx[4] = {0, 0, 0, 0};
   for (int q0 = 0; q0 < nq; q0 += LPG * QC) {
@@ -119,7 +126,6 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   int v[4];
   // symmetric weights: 2 * raw - wmax * (activation sum), written without a branch (shift 0 and weight
   // range 0 for the plain result)
-  const int sym_sh = p.sym ? 1 : 0, sym_w = p.sym ? p.wmax : 0;
 #pragma unroll
   for (int o = 0; o < 4; ++o) v[o] = (acc[o] << sym_sh) - sym_w * sx[ACT_A ? 0 : o];
   // butterfly over the eight lanes of a group with data-parallel-primitive adds: lane ^ 1 and lane ^ 2
@@ -136,8 +142,8 @@ __global__ __launch_bounds__(256) void apnn_valu_direct_kernel(const KParams p) 
   const int m01 = (l4 & 1) ? v[1] : v[0], m23 = (l4 & 1) ? v[3] : v[2];
   const int mine = (l4 & 2) ? m23 : m01;
 
-  if (p.epi == APNN_EPI_INT32) {
-    if (live && l < 4) reinterpret_cast<int *>(p.out)[(long long)a * p.rowsB + b + l] = mine;
+  if (epi == APNN_EPI_INT32) {
+    if (live && l < 4) out_i32[(long long)a * p.rowsB + b + l] = mine;
     return;
   }
   if constexpr (LPG == 4) {
