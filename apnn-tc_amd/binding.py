@@ -4,7 +4,8 @@ import os
 import subprocess
 
 __all__ = [
-    "LIB_PATH", "lib", "build", "Epilogue", "GemmDesc", "ConvDesc", "ApnnError", "check",
+    "LIB_PATH", "lib", "build", "Epilogue", "GemmDesc", "ConvDesc", "Plan", "ApnnError", "check",
+    "KERNEL_VALU_TILE", "KERNEL_VALU_DIRECT", "KERNEL_MFMA_FP4", "KERNEL_MFMA_I8", "KERNEL_PATCH_FP4",
     "EPI_INT32", "EPI_LOWBITS", "EPI_BN", "POOL_NONE", "POOL_AVG2X2", "POOL_MAX2X2",
     "PATH_AUTO", "PATH_VALU", "PATH_MFMA", "PATH_MFMA_I8", "PATH_MFMA_PATCH", "WEIGHT_UNSIGNED", "WEIGHT_SYMMETRIC",
     "OK", "EINVAL", "ENULL", "EALIGN", "EUNSUPPORTED", "DECLARED_SYMBOLS",
@@ -41,18 +42,26 @@ class ConvDesc(ctypes.Structure):
                 ("path", _ci)]
 
 
+class Plan(ctypes.Structure):
+    _fields_ = [("path", _ci), ("kernel", _ci), ("tile", _ci), ("tile_rows", _ci), ("tile_cols", _ci),
+                ("split_k", _ci), ("workgroups", ctypes.c_longlong), ("patch_pixels", _ci), ("fp4_exact", _ci)]
+
+
+KERNEL_VALU_TILE, KERNEL_VALU_DIRECT, KERNEL_MFMA_FP4, KERNEL_MFMA_I8, KERNEL_PATCH_FP4 = 0, 1, 2, 3, 4
+
 _GEMM_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp]
 _CONV_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 
 _GEMM_NAMES = ["apmm_w1a2", "apmm_w1a3", "apmm_w1a4", "apmm_w2a2", "apmm_w1a8", "apmm_w2a8", "apmm_w4a4", "apmm_w1a1",
                "apmm_w1a2_decompose", "apmm_w1a3_decompose", "apmm_w1a4_decompose", "apmm_w2a2_decompose"]
 _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2", "apconv_w1a5", "apconv_w2a6",
-               "APConv_w2a8_pack",
+               "apconv_w1a8", "apconv_w2a8", "APConv_w2a8_pack", "APConv_w2a8_pack_pool",
                "APConv_w1a2_pack", "APConv_w1a3_pack", "APConv_w1a4_pack", "APConv_w2a2_pack",
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
 DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
                                                 "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
                                                 "apnn_conv_i8_bn_pack", "apnn_pool_planes", "apnn_quantize_pack", "apnn_fold_bn", "apnn_conv_pair",
+                                                "apnn_gemm_plan", "apnn_conv_plan",
                                                 "apnn_device_cus", "apnn_version"]
 
 
@@ -102,6 +111,10 @@ def lib():
         L.apnn_gemm.restype = _ci
         L.apnn_conv.argtypes = [ctypes.POINTER(ConvDesc), _vp]
         L.apnn_conv.restype = _ci
+        L.apnn_gemm_plan.argtypes = [ctypes.POINTER(GemmDesc), ctypes.POINTER(Plan)]
+        L.apnn_gemm_plan.restype = _ci
+        L.apnn_conv_plan.argtypes = [ctypes.POINTER(ConvDesc), ctypes.POINTER(Plan)]
+        L.apnn_conv_plan.restype = _ci
         L.apnn_conv_pair.argtypes = [ctypes.POINTER(ConvDesc), ctypes.POINTER(ConvDesc), _vp]
         L.apnn_conv_pair.restype = _ci
         L.apnn_pack_bits.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]

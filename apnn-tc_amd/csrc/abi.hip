@@ -100,22 +100,50 @@ void fill_epilogue(KParams &p, const apnn_epilogue &e, void *out, long long out_
 
 typedef hipError_t (*valu_fn)(int, int, const KParams &, hipStream_t);
 
+// Matrix-core kernels: both operand encodings for the four benchmark precisions; FP4 only (a reduced
+// tile set, see mfma_tile_enabled) for the wider precisions of the reference tree.
 valu_fn mfma_gemm_fn(int wb, int xb, bool i8) {
   if (wb == 1 && xb == 2) return i8 ? apnn::mfma_gemm_1_2_x : apnn::mfma4_gemm_1_2_x;
   if (wb == 1 && xb == 3) return i8 ? apnn::mfma_gemm_1_3_x : apnn::mfma4_gemm_1_3_x;
   if (wb == 1 && xb == 4) return i8 ? apnn::mfma_gemm_1_4_x : apnn::mfma4_gemm_1_4_x;
   if (wb == 2 && xb == 2) return i8 ? apnn::mfma_gemm_2_2_x : apnn::mfma4_gemm_2_2_x;
+  if (i8) return nullptr;
+  if (wb == 4 && xb == 4) return apnn::mfma4_gemm_4_4_x;
+  if (wb == 1 && xb == 8) return apnn::mfma4_gemm_1_8_x;
+  if (wb == 2 && xb == 8) return apnn::mfma4_gemm_2_8_x;
   return nullptr;
 }
 
-// the int8 core is built for the GEMM entry points only
 valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
+  if (xb == 2 && wb == 1) return i8 ? apnn::mfma_conv_2_1_x : apnn::mfma4_conv_2_1_x;
+  if (xb == 3 && wb == 1) return i8 ? apnn::mfma_conv_3_1_x : apnn::mfma4_conv_3_1_x;
+  if (xb == 4 && wb == 1) return i8 ? apnn::mfma_conv_4_1_x : apnn::mfma4_conv_4_1_x;
+  if (xb == 2 && wb == 2) return i8 ? apnn::mfma_conv_2_2_x : apnn::mfma4_conv_2_2_x;
   if (i8) return nullptr;
-  if (xb == 2 && wb == 1) return apnn::mfma4_conv_2_1_x;
-  if (xb == 3 && wb == 1) return apnn::mfma4_conv_3_1_x;
-  if (xb == 4 && wb == 1) return apnn::mfma4_conv_4_1_x;
-  if (xb == 2 && wb == 2) return apnn::mfma4_conv_2_2_x;
+  if (xb == 8 && wb == 1) return apnn::mfma4_conv_8_1_x;
+  if (xb == 8 && wb == 2) return apnn::mfma4_conv_8_2_x;
   return nullptr;
+}
+
+// The FP4 matrix-core kernels accumulate in fp32: every partial sum is a multiple of 1/4 and stays
+// exact while the largest possible result, K * (2^w - 1) * (2^a - 1), is below 2^24.
+bool fp4_exact(long long kwords, int wb, int xb) {
+  return kwords * 32 * ((1LL << wb) - 1) * ((1LL << xb) - 1) < (1LL << 24);
+}
+
+// Reports a kernel choice instead of launching it (apnn_gemm_plan / apnn_conv_plan).
+int fill_plan(apnn_plan *plan, int path, int kernel, int tile, int tr, int tc, int split_k, const KParams &p,
+              int patch_pixels_, bool f4ok) {
+  plan->path = path;
+  plan->kernel = kernel;
+  plan->tile = tile;
+  plan->tile_rows = tr;
+  plan->tile_cols = tc;
+  plan->split_k = split_k;
+  plan->workgroups = tr > 0 && tc > 0 ? (long long)((p.rowsA + tr - 1) / tr) * ((p.rowsB + tc - 1) / tc) : 0;
+  plan->patch_pixels = patch_pixels_;
+  plan->fp4_exact = f4ok ? 1 : 0;
+  return APNN_OK;
 }
 
 // what the register-only kernel (valu_direct_kernel.h) handles
@@ -202,7 +230,7 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, bool wide = false) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
@@ -213,7 +241,20 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
   auto fill = [&](int t) {
     return (double)rowsA * rowsB / ((double)ntiles(t) * apnn::kMfmaTileA[t] * apnn::kMfmaTileB[t]);
   };
-  if (i8) {  // int8 core: 256x128, 128x128 and 64x64 are built
+  if (wide) {  // more than five planes in all: 128x128, 64x64 and the 32x32 split-K tile are built
+    if (conv && vw != 4) return 2;
+    if (KW >= 32 && ntiles(4) <= 256) return 4;
+    return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
+  }
+  if (i8 && conv) {  // int8 core, convolution: 128x256, 128x128, 128x64, 64x64, 32x32 split-K (128-bit loads)
+    if (vw != 4) return 2;
+    if (KW >= 32 && ntiles(4) <= 256) return 4;
+    if (rowsB > 64 && ntiles(7) >= cus && fill(7) >= 0.8) return 7;
+    if (rowsB > 64 && ntiles(1) >= cus && fill(1) >= 0.8) return 1;
+    if (rowsB <= 64 && ntiles(3) >= cus) return 3;
+    return 2;
+  }
+  if (i8) {  // int8 core, GEMM entry points: 256x128, 128x128 and 64x64 are built
     if (ntiles(6) >= cus && fill(6) >= 0.8) return 6;
     return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
   }
@@ -242,7 +283,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8) {
 
 int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB > 5);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
@@ -281,7 +322,28 @@ valu_fn valu_conv_fn(int xb, int wb) {
   return apnn::valu_conv_any_x;
 }
 
-int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
+constexpr int kValuTileA[apnn::TILE_COUNT] = {64, 32, 16, 16};
+constexpr int kValuTileB[apnn::TILE_COUNT] = {64, 32, 32, 16};
+
+// the any-precision VALU instantiation has one 32x32 tile
+int plan_valu(apnn_plan *plan, int tile, bool any, const KParams &p, bool f4ok) {
+  const int t = any ? apnn::TILE_32x32 : tile;
+  return fill_plan(plan, APNN_PATH_VALU, APNN_KERNEL_VALU_TILE, t, kValuTileA[t], kValuTileB[t], 1, p, 0, f4ok);
+}
+
+int plan_direct(apnn_plan *plan, const KParams &p, bool f4ok) {
+  // one wave per row and 32 columns, four waves per work-group
+  return fill_plan(plan, APNN_PATH_VALU, APNN_KERNEL_VALU_DIRECT, apnn::TILE_DIRECT, 1, 128, 1, p, 0, f4ok);
+}
+
+int plan_mfma(apnn_plan *plan, bool i8, int tile, const KParams &p, bool f4ok) {
+  const bool split = tile == 4 || tile == 5;
+  return fill_plan(plan, i8 ? APNN_PATH_MFMA_I8 : APNN_PATH_MFMA, i8 ? APNN_KERNEL_MFMA_I8 : APNN_KERNEL_MFMA_FP4, tile,
+                   apnn::kMfmaTileA[tile], apnn::kMfmaTileB[tile], split ? 4 : 1, p, 0, f4ok);
+}
+
+// plan != nullptr: report the choice, launch nothing
+int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = nullptr) {
   if (d == nullptr) return APNN_ENULL;
   int rc;
   if ((rc = check_dev_ptr(d->W)) || (rc = check_dev_ptr(d->X)) || (rc = check_dev_ptr(d->D))) return rc;
@@ -308,24 +370,38 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream) {
   int tile;
   p.planesA = d->wb;
   p.planesB = d->xb;
+  const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
+  if (path == APNN_PATH_MFMA && !f4ok) return APNN_EUNSUPPORTED;  // fp32 accumulation would round
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
-    valu_fn fn = mfma_gemm_fn(d->wb, d->xb, path == APNN_PATH_MFMA_I8);
+    // AUTO: FP4 operands while their fp32 accumulation is exact, the int8 core (int32 accumulate) beyond
+    const bool i8 = path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && !f4ok);
+    valu_fn fn = mfma_gemm_fn(d->wb, d->xb, i8);
     if (fn != nullptr) {
-      if ((rc = pick_mfma_tile(tile_pin, p, false, 4, path == APNN_PATH_MFMA_I8, &tile))) return rc;
+      if ((rc = pick_mfma_tile(tile_pin, p, false, 4, i8, &tile))) return rc;
+      if (plan != nullptr) {
+        // a pinned tile that is not built is reported by the launcher; mirror that here
+        return apnn::mfma_tile_enabled(i8 ? apnn::CORE_I8 : apnn::CORE_F4, false, 4, tile, d->wb, d->xb)
+                   ? plan_mfma(plan, i8, tile, p, f4ok)
+                   : APNN_EUNSUPPORTED;
+      }
       return from_hip(fn(4, tile, p, stream));
     }
     if (path != APNN_PATH_AUTO) return APNN_EUNSUPPORTED;  // precisions without a matrix-core kernel
   }
   valu_fn fn = valu_gemm_fn(d->wb, d->xb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
-  const bool direct_ok = fn != apnn::valu_gemm_any_x && direct_kernel_serves(p);
-  if (tile_pin == apnn::TILE_DIRECT + 1)  // register-only kernel
-    return direct_ok ? from_hip(fn(4, apnn::TILE_DIRECT, p, stream)) : APNN_EUNSUPPORTED;
+  const bool any = fn == apnn::valu_gemm_any_x;
+  const bool direct_ok = !any && direct_kernel_serves(p);
+  if (tile_pin == apnn::TILE_DIRECT + 1) {  // register-only kernel
+    if (!direct_ok) return APNN_EUNSUPPORTED;
+    return plan != nullptr ? plan_direct(plan, p, f4ok) : from_hip(fn(4, apnn::TILE_DIRECT, p, stream));
+  }
   // small, latency-bound problems (the M = 64 sweep): one round of loads, no LDS, no barrier
   if (tile_pin == 0 && direct_ok && p.KW <= 64 && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
-    return from_hip(fn(4, apnn::TILE_DIRECT, p, stream));
+    return plan != nullptr ? plan_direct(plan, p, f4ok) : from_hip(fn(4, apnn::TILE_DIRECT, p, stream));
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
+  if (plan != nullptr) return plan_valu(plan, tile, any, p, f4ok);
   return (int)fn(4, tile, p, stream);
 }
 
@@ -391,12 +467,13 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   return APNN_OK;
 }
 
-int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
+int run_conv(const apnn_conv_desc *d, hipStream_t stream, apnn_plan *plan = nullptr) {
   KParams p{};
   int vw = 1, rc, tile;
   if ((rc = build_conv_params(d, p, &vw))) return rc;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
   const int Ho = p.Ho, Wo = p.Wo;
+  const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
   // A filter that spans the whole stored input map (fully connected layer): every output pixel is one
   // image, whose im2col row is the image itself -- a plain GEMM over rows of KW words.  With few
   // outputs (small batch) the layer streams its weights; the register-only kernel serves it.
@@ -404,26 +481,39 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   {
     valu_fn vf = valu_conv_fn(d->xb, d->wb);
     const bool fc_direct_ok = fc_shape && vf != nullptr && vf != apnn::valu_conv_any_x && direct_kernel_serves(p);
-    if (path == APNN_PATH_VALU && tile_pin == apnn::TILE_DIRECT + 1)
-      return fc_direct_ok ? from_hip(vf(vw, apnn::TILE_DIRECT, p, stream)) : APNN_EUNSUPPORTED;
+    if (path == APNN_PATH_VALU && tile_pin == apnn::TILE_DIRECT + 1) {
+      if (!fc_direct_ok) return APNN_EUNSUPPORTED;
+      return plan != nullptr ? plan_direct(plan, p, f4ok) : from_hip(vf(vw, apnn::TILE_DIRECT, p, stream));
+    }
     if (path == APNN_PATH_AUTO && tile_pin == 0 && fc_direct_ok && (long long)p.rowsA * p.rowsB <= 2 * 256LL * 256)
-      return from_hip(vf(vw, apnn::TILE_DIRECT, p, stream));
+      return plan != nullptr ? plan_direct(plan, p, f4ok) : from_hip(vf(vw, apnn::TILE_DIRECT, p, stream));
   }
-  if (path == APNN_PATH_MFMA_PATCH || path == APNN_PATH_AUTO) {
+  // fp32 accumulation of the FP4 kernels would round: pinned FP4 paths refuse, AUTO moves on
+  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_PATCH) && !f4ok) return APNN_EUNSUPPORTED;
+  if (path == APNN_PATH_MFMA_PATCH || (path == APNN_PATH_AUTO && f4ok)) {
     patch_fn pf = patch_conv_fn(d->xb, d->wb);
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
     if (pt >= 0) {
       p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
       p.magicPW = magic_of(p.PWs);
       p.magicPH = magic_of(p.PHs);
+      if (plan != nullptr)
+        return fill_plan(plan, APNN_PATH_MFMA_PATCH, APNN_KERNEL_PATCH_FP4, pt, apnn::kPatchTileRows[pt],
+                         apnn::kPatchTileCols[pt], 1, p, p.patch_cap, f4ok);
       return from_hip(pf(pt, p, stream));
     }
     if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;
   }
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
-    valu_fn fn = mfma_conv_fn(d->xb, d->wb, path == APNN_PATH_MFMA_I8);
+    const bool i8 = path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && !f4ok);
+    valu_fn fn = mfma_conv_fn(d->xb, d->wb, i8);
     if (fn != nullptr) {
-      if ((rc = pick_mfma_tile(tile_pin, p, true, vw, false, &tile))) return rc;
+      if ((rc = pick_mfma_tile(tile_pin, p, true, vw, i8, &tile))) return rc;
+      if (plan != nullptr) {
+        return apnn::mfma_tile_enabled(i8 ? apnn::CORE_I8 : apnn::CORE_F4, true, vw, tile, d->xb, d->wb)
+                   ? plan_mfma(plan, i8, tile, p, f4ok)
+                   : APNN_EUNSUPPORTED;
+      }
       return from_hip(fn(vw, tile, p, stream));
     }
     if (path != APNN_PATH_AUTO) return APNN_EUNSUPPORTED;
@@ -431,6 +521,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream) {
   valu_fn fn = valu_conv_fn(d->xb, d->wb);
   if (fn == nullptr) return APNN_EUNSUPPORTED;
   if ((rc = pick_valu_tile(tile_pin, p, d->epi.mode != APNN_EPI_INT32, &tile))) return rc;
+  if (plan != nullptr) return plan_valu(plan, tile, fn == apnn::valu_conv_any_x, p, f4ok);
   return (int)fn(vw, tile, p, stream);
 }
 
@@ -451,7 +542,8 @@ int run_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, hipStream_t 
   valu_fn fn = mfma_conv_fn(a->xb, a->wb, false);
   const bool fusable = fn != nullptr && plain_bn(a->epi) && plain_bn(b->epi) && a->epi.out_bits == b->epi.out_bits &&
                        (a->path & 0xffff) == APNN_PATH_AUTO && (b->path & 0xffff) == APNN_PATH_AUTO &&
-                       auto_prefers_mfma(pa) && a->O != b->O;
+                       auto_prefers_mfma(pa) && a->O != b->O && fp4_exact(pa.KW, a->wb, a->xb) &&
+                       fp4_exact(pb.KW, b->wb, b->xb);
   if (!fusable) {
     if ((rc = run_conv(a, stream))) return rc;
     return run_conv(b, stream);
@@ -550,7 +642,10 @@ APNN_DEF_CONV(apconv_w1a4, 1, 4, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w2a2, 2, 2, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w1a5, 1, 5, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(apconv_w2a6, 2, 6, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w1a8, 1, 8, APNN_EPI_INT32, APNN_POOL_NONE)
+APNN_DEF_CONV(apconv_w2a8, 2, 8, APNN_EPI_INT32, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w2a8_pack, 2, 8, APNN_EPI_LOWBITS, APNN_POOL_NONE)
+APNN_DEF_CONV(APConv_w2a8_pack_pool, 2, 8, APNN_EPI_LOWBITS, APNN_POOL_AVG2X2)
 APNN_DEF_CONV(APConv_w1a2_pack, 1, 2, APNN_EPI_LOWBITS, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w1a3_pack, 1, 3, APNN_EPI_LOWBITS, APNN_POOL_NONE)
 APNN_DEF_CONV(APConv_w1a4_pack, 1, 4, APNN_EPI_LOWBITS, APNN_POOL_NONE)
@@ -561,6 +656,12 @@ APNN_DEF_CONV(APConv_w2a2_pack_pool, 2, 2, APNN_EPI_LOWBITS, APNN_POOL_AVG2X2)
 
 int apnn_gemm(const apnn_gemm_desc *d, apnn_stream_t s) { return run_gemm(d, static_cast<hipStream_t>(s)); }
 int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s) { return run_conv(d, static_cast<hipStream_t>(s)); }
+int apnn_gemm_plan(const apnn_gemm_desc *d, apnn_plan *plan) {
+  return plan == nullptr ? APNN_ENULL : run_gemm(d, nullptr, plan);
+}
+int apnn_conv_plan(const apnn_conv_desc *d, apnn_plan *plan) {
+  return plan == nullptr ? APNN_ENULL : run_conv(d, nullptr, plan);
+}
 int apnn_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, apnn_stream_t s) {
   return run_conv_pair(a, b, static_cast<hipStream_t>(s));
 }

@@ -28,6 +28,15 @@ APNN_DECL_MFMA(gemm, 1, 2)
 APNN_DECL_MFMA(gemm, 1, 3)
 APNN_DECL_MFMA(gemm, 1, 4)
 APNN_DECL_MFMA(gemm, 2, 2)
+APNN_DECL_MFMA(conv, 2, 1)
+APNN_DECL_MFMA(conv, 3, 1)
+APNN_DECL_MFMA(conv, 4, 1)
+APNN_DECL_MFMA(conv, 2, 2)
+APNN_DECL_MFMA4(gemm, 4, 4)
+APNN_DECL_MFMA4(gemm, 1, 8)
+APNN_DECL_MFMA4(gemm, 2, 8)
+APNN_DECL_MFMA4(conv, 8, 1)
+APNN_DECL_MFMA4(conv, 8, 2)
 APNN_DECL_MFMA4(gemm, 1, 2)
 APNN_DECL_MFMA4(gemm, 1, 3)
 APNN_DECL_MFMA4(gemm, 1, 4)
@@ -45,10 +54,40 @@ APNN_DECL_PATCH(2, 2)
 #undef APNN_DECL_PATCH
 #undef APNN_DECL_MFMA4
 
+// operand encodings of the matrix-core kernels (mfma_kernel.h)
+enum { CORE_I8 = 0, CORE_F4 = 1 };
+
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
 constexpr int kMfmaTileCount = 8;
 constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128};
 constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256};
+
+enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
+                MT_256x128 = 6, MT_128x256 = 7, MT_COUNT = 8 };
+
+// Which (core, family, load width, tile, plane counts) combinations are built.  Every kernel
+// instantiation costs seconds of compile time, so only the shapes the dispatcher can choose are kept:
+//   int8 core : GEMM entry points 256x128, 128x128, 64x64; convolution with 128-bit loads 128x256,
+//               128x128, 128x64, 64x64 and the 32x32 split-K tile, with narrower loads 64x64 only
+//   FP4 core  : GEMM: all but 256x256 / 128x256;  convolution: all but 256x256 / 256x128, and only
+//               the two small tiles when the stored channel count allows 32-bit loads only;
+//               more than five planes in all (w4a4, w1a8, w2a8): 128x128, 64x64, 32x32 split-K
+//               (convolution with narrower loads: 64x64 only); the int8 core is not built for those.
+constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile, int pa, int pb) {
+  if (pa + pb > 5) {
+    if (core == CORE_I8) return false;
+    if (conv && vw != 4) return tile == MT_64x64;
+    return tile == MT_128x128 || tile == MT_64x64 || tile == MT_32x32_K4;
+  }
+  if (core == CORE_I8) {
+    if (!conv) return tile == MT_128x128 || tile == MT_64x64 || tile == MT_256x128;
+    if (vw != 4) return tile == MT_64x64;
+    return tile == MT_128x256 || tile == MT_128x128 || tile == MT_128x64 || tile == MT_64x64 || tile == MT_32x32_K4;
+  }
+  if (!conv) return tile != MT_256x256 && tile != MT_128x256;
+  if (vw == 1) return tile == MT_64x64 || tile == MT_32x32_K4;
+  return tile != MT_256x256 && tile != MT_256x128;
+}
 
 // tile shapes of the patch-resident convolution kernel, index = enum PatchTile in patch_conv_kernel.h
 constexpr int kPatchTileCount = 5;

@@ -33,6 +33,7 @@
 
 #include <type_traits>
 
+#include "dispatch.h"
 #include "epilogue.h"
 #include "kparams.h"
 #include "valu_kernel.h"  // load_words, fast_div
@@ -43,8 +44,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-
-enum { CORE_I8 = 0, CORE_F4 = 1 };
 
 // FP4 operand for digit D (planes 2D and, if present, 2D+1) of a P-plane row word: nibble c of
 // result word t is the digit of element 4c + t.
@@ -1018,10 +1017,10 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
 }
 
-constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
+constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
   const size_t ld = WA * WB == 1 ? 33 : (conv && FA * FB <= 2 && vw == 4) ? 17 : 9;  // KC + 1, see the kernel
-  // split-K tiles with 128-bit loads stage nothing (operands go from global memory to registers)
-  const size_t stage = WA * WB == 1 && vw == 4
+  // FP4 split-K tiles with 128-bit loads stage nothing (operands go from global memory to registers)
+  const size_t stage = core == CORE_F4 && WA * WB == 1 && vw == 4
                            ? 0
                            : 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
   const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
@@ -1032,7 +1031,7 @@ constexpr size_t mfma_smem_bytes(int PA, int PB, int FA, int FB, int WA, int WB,
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr size_t smem_bytes = mfma_smem_bytes(PA, PB, FA, FB, WA, WB, CONV, VW);
+  constexpr size_t smem_bytes = mfma_smem_bytes(CORE, PA, PB, FA, FB, WA, WB, CONV, VW);
   constexpr int OCC_FIT = (int)((160 * 1024) / smem_bytes);
   constexpr int OCC = OCC_FIT < 1 ? 1 : (OCC_FIT < OCC_WANTED ? OCC_FIT : OCC_WANTED);
   static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
@@ -1053,24 +1052,9 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
-                MT_256x128 = 6, MT_128x256 = 7, MT_COUNT = 8 };
-
-// Which (core, family, load width, tile) combinations are built.  Every kernel instantiation costs
-// seconds of compile time, so only the shapes the dispatcher can choose are kept:
-//   int8 core : GEMM entry points only (the second matrix-core variant, for comparison runs)
-//   FP4 core  : GEMM: all but 256x256 / 128x256;  convolution: all but 256x256 / 256x128, and only
-//               the two small tiles when the stored channel count allows 32-bit loads only.
-constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile) {
-  if (core == CORE_I8) return !conv && (tile == MT_128x128 || tile == MT_64x64 || tile == MT_256x128);
-  if (!conv) return tile != MT_256x256 && tile != MT_128x256;
-  if (vw == 1) return tile == MT_64x64 || tile == MT_32x32_K4;
-  return tile != MT_256x256 && tile != MT_256x128;
-}
-
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC, int TILE>
 inline hipError_t launch_mfma_if_enabled(const KParams &p, hipStream_t stream) {
-  if constexpr (mfma_tile_enabled(CORE, CONV, VW, TILE)) {
+  if constexpr (mfma_tile_enabled(CORE, CONV, VW, TILE, PA, PB)) {
     return launch_mfma<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>(p, stream);
   } else {
     return hipErrorNotSupported;

@@ -51,7 +51,8 @@ int apmm_w2a2(const void *W, const void *X, int *D, int M, int N, int K, int wb,
 /* Further precisions of the reference tree, same definition and constraints: apmm_w1a8
  * (LIB/77_bmmaTensorCoreGemm.cu:80), apmm_w2a8 (LIB/76_bmmaTensorCoreGemm.cuh:80-82), apmm_w4a4
  * (LIB/83_bmmaTensorCoreGemm.cu:80), apmm_w1a1 (LIB/84_bmmaTensorCoreGemm.cu:80).  Any other (w, a) up to
- * 8 bits each is served by apnn_gemm / apnn_conv.  These run on the any-precision VALU kernel. */
+ * 8 bits each is served by apnn_gemm / apnn_conv.  w4a4, w1a8 and w2a8 have FP4 matrix-core kernels
+ * (digit pairs weighted through the block scale) besides the any-precision VALU kernel. */
 int apmm_w1a8(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
 int apmm_w2a8(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
 int apmm_w4a4(const void *W, const void *X, int *D, int M, int N, int K, int wb, int xb, apnn_stream_t s);
@@ -77,6 +78,9 @@ int apconv_w2a2(const void *W, const void *X, int *Output, int Height, int Width
 /* compute_conv_imma at w1a5 (LIB/61_bmmaTensorCoreGemm.cu:58, LIB/62) and w2a6 (LIB/63_bmmaTensorCoreGemm.cu:58). */
 int apconv_w1a5(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 int apconv_w2a6(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+/* compute_conv_imma at w1a8 (LIB/55_bmmaTensorCoreGemm.cu:58, LIB/56) and w2a8 (LIB/57_bmmaTensorCoreGemm.cu:58, LIB/58). */
+int apconv_w1a8(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+int apconv_w2a8(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 
 /* Convolution, then low-bit planes of the result: Output:[a][H][W][COUT/32].
  * Replace APConv_w1a2_pack (LIB/67h:60-325) and APConv_w2a2_pack (LIB/70_bmmaTensorCoreGemm.cu:58).
@@ -94,6 +98,8 @@ int APConv_w2a8_pack(const void *W, const void *X, int *Output, int Height, int 
  * and APConv_w2a2_pack_pool (LIB/69_bmmaTensorCoreGemm.cuh:60).  Requires even Height and Width. */
 int APConv_w1a2_pack_pool(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 int APConv_w2a2_pack_pool(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
+/* APConv_w2a8_pack_pool (LIB/75_bmmaTensorCoreGemm.cu:58): Output:[8][H/2][W/2][COUT/32]. */
+int APConv_w2a8_pack_pool(const void *W, const void *X, int *Output, int Height, int Width, int CIN, int COUT, apnn_stream_t s);
 
 /* ---- general descriptor entry points ------------------------------------------------------- */
 
@@ -105,7 +111,9 @@ enum { APNN_POOL_NONE = 0,
        APNN_POOL_MAX2X2 = 2 };/* max over the 2x2 window of the quantized codes                     */
 enum { APNN_PATH_AUTO = 0,
        APNN_PATH_VALU = 1,     /* v_and + v_bcnt popcount on packed words                           */
-       APNN_PATH_MFMA = 2,     /* planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4      */
+       APNN_PATH_MFMA = 2,     /* planes expanded to FP4 operands of v_mfma_f32_32x32x64_f8f6f4; fp32
+                                  accumulation, exact while K*(2^wb-1)*(2^xb-1) < 2^24: beyond that a
+                                  pinned FP4 path returns APNN_EUNSUPPORTED and AUTO uses the int8 core   */
        APNN_PATH_MFMA_I8 = 3,  /* planes expanded to int8 operands of v_mfma_i32_32x32x32_i8         */
        APNN_PATH_MFMA_PATCH = 4 };/* convolution only: FP4 matrix-core path with the tile's input patch
                                   expanded once into LDS and read in place by every filter tap;
@@ -171,6 +179,27 @@ typedef struct apnn_conv_desc {
   int path;
 } apnn_conv_desc;
 int apnn_conv(const apnn_conv_desc *d, apnn_stream_t s);
+
+/* What apnn_gemm / apnn_conv would launch for a descriptor: same validation and kernel choice, nothing
+ * is enqueued and no buffer is touched (no counterpart in the reference, whose kernels are picked at
+ * compile time).  For tuning, and for checking the dispatcher without a device. */
+enum { APNN_KERNEL_VALU_TILE = 0,   /* LDS-tiled popcount kernel                                     */
+       APNN_KERNEL_VALU_DIRECT = 1, /* register-only popcount kernel (small GEMMs, FC layers)         */
+       APNN_KERNEL_MFMA_FP4 = 2,
+       APNN_KERNEL_MFMA_I8 = 3,
+       APNN_KERNEL_PATCH_FP4 = 4 };
+typedef struct apnn_plan {
+  int path;              /* APNN_PATH_* taken (never AUTO) */
+  int kernel;            /* APNN_KERNEL_* */
+  int tile;              /* tile index within the kernel family (the value APNN_PATH_TILE pins) */
+  int tile_rows, tile_cols; /* outputs per work-group: slow x fast output index */
+  int split_k;           /* waves of a work-group that share one output block */
+  long long workgroups;
+  int patch_pixels;      /* APNN_KERNEL_PATCH_FP4: padded-frame pixels a work-group stages, else 0 */
+  int fp4_exact;         /* 1: fp32 accumulation of FP4 operands is exact for this reduction length */
+} apnn_plan;
+int apnn_gemm_plan(const apnn_gemm_desc *d, apnn_plan *plan);
+int apnn_conv_plan(const apnn_conv_desc *d, apnn_plan *plan);
 
 /* Bit-plane packer with the layout of Bit_compression (NN/kernel.cuh:46-77):
  * values:[rows][C] uint32 codes -> planes:[bits][rows][cpad/32], channel c at bit 31-c%32,

@@ -304,6 +304,7 @@ void oracle_unpack_bits(const uint32_t *planes, uint32_t *values, int rows, int 
 void oracle_conv_i8(const int8_t *Wt, const int8_t *X, int32_t *O,
                     int B, int H, int Wd, int C, int cout, int R, int S, int stride, int pad) {
   const int Ho = (H + 2 * pad - R) / stride + 1, Wo = (Wd + 2 * pad - S) / stride + 1;
+#pragma omp parallel for collapse(2) schedule(static)
   for (int b = 0; b < B; b++)
     for (int oy = 0; oy < Ho; oy++)
       for (int ox = 0; ox < Wo; ox++)

@@ -193,6 +193,28 @@ def unpack_planes_lsb(planes):
     return (bits * weights).sum(0)
 
 
+def gemm_column_sums(W, X, chunk=1024):
+    """sum_m D[m][n] of the unsigned GEMM D = wvalue . xvalue^T, without forming D:
+    (sum_m wvalue[m][:]) . xvalue[n][:].  Row chunks bound the memory; float64 products are exact here
+    (every partial sum is far below 2^53)."""
+    W, X = np.asarray(W, np.uint32), np.asarray(X, np.uint32)
+    shifts = np.arange(32, dtype=np.uint32)
+
+    def bits_of(plane_rows):                                        # [rows][words] -> [rows][32*words] uint8
+        return ((plane_rows[..., None] >> shifts) & 1).astype(np.uint8).reshape(plane_rows.shape[0], -1)
+
+    wsum = np.zeros(W.shape[2] * 32, np.int64)
+    for p in range(W.shape[0]):
+        for r0 in range(0, W.shape[1], chunk):
+            wsum += bits_of(W[p, r0:r0 + chunk]).sum(0, dtype=np.int64) << p
+    wsum_f = wsum.astype(np.float64)
+    out = np.zeros(X.shape[1], np.float64)
+    for p in range(X.shape[0]):
+        for r0 in range(0, X.shape[1], chunk):
+            out[r0:r0 + chunk] += (bits_of(X[p, r0:r0 + chunk]).astype(np.float64) @ wsum_f) * float(1 << p)
+    return out.astype(np.int64)
+
+
 def random_planes(rng, planes, rows, words):
     return rng.integers(0, 2 ** 32, size=(planes, rows, words), dtype=np.uint64).astype(np.uint32)
 

@@ -96,12 +96,14 @@ def test_combinations_that_are_not_built_are_reported():
     L = A.lib()
     good = 0x1000
     c = A.ConvDesc(W=good, X=good, O=good, batch=1, H=8, Wd=8, cin_pad=128, COUT=64, R=3, S=3, stride=1, pad=1,
-                   wb=1, xb=2, path=A.PATH_MFMA_I8)
-    assert L.apnn_conv(ctypes.byref(c), None) == A.EUNSUPPORTED          # int8 core: GEMM entry points only
+                   wb=1, xb=2, path=A.PATH_MFMA_I8 | ((0 + 1) << 8))
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EUNSUPPORTED          # int8 convolution has no 256x256 tile
+    c.wb, c.xb, c.path = 1, 8, A.PATH_MFMA_I8
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EUNSUPPORTED          # wide precisions: FP4 core only
     g = A.GemmDesc(W=good, X=good, D=good, M=64, N=128, K=128, wb=1, xb=2, path=A.PATH_MFMA | (1 << 8))
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # FP4 GEMM has no 256x256 tile
     g.wb, g.xb, g.path = 3, 5, A.PATH_MFMA
-    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # matrix-core kernels: w1a2 / w1a3 / w1a4 / w2a2
+    assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # no matrix-core kernel for w3a5
     g.path = A.PATH_MFMA_PATCH
     assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED          # convolution only
     g.wb, g.xb, g.path = 9, 2, A.PATH_AUTO
@@ -147,3 +149,121 @@ def test_fold_bn_matches_double_precision_brute_force():
     bad = np.zeros(4, np.float32)
     assert L.apnn_fold_bn(None, p(bad), p(bad), p(bad), eps, 1.0, 1.0, 4, 2, p(thr), p(flip)) == A.ENULL
     assert L.apnn_fold_bn(p(bad), p(bad), p(bad), p(bad), eps, 1.0, 0.0, 4, 2, p(thr), p(flip)) == A.EINVAL
+
+
+def _plan_gemm(**kw):
+    g = A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, **kw)
+    plan = A.Plan()
+    rc = A.lib().apnn_gemm_plan(ctypes.byref(g), ctypes.byref(plan))
+    return rc, plan
+
+
+def _plan_conv(**kw):
+    c = A.ConvDesc(W=0x1000, X=0x1000, O=0x1000, **kw)
+    plan = A.Plan()
+    rc = A.lib().apnn_conv_plan(ctypes.byref(c), ctypes.byref(plan))
+    return rc, plan
+
+
+def test_fp4_accumulation_guard():
+    """The FP4 matrix-core kernels accumulate in fp32, exact while K*(2^w-1)*(2^a-1) < 2^24.  Beyond that
+    bound the library's own choice moves to the int8 core (int32 accumulate) and a pinned FP4 path is
+    refused -- decided on the host, before any launch."""
+    L = A.lib()
+    for wb, xb in [(1, 2), (1, 3), (1, 4), (2, 2)]:
+        span = (2 ** wb - 1) * (2 ** xb - 1)
+        k_ok = ((2 ** 24 - 1) // span) // 128 * 128              # largest exact K
+        k_bad = k_ok + 128
+        assert k_ok * span < 2 ** 24 <= k_bad * span
+        rc, plan = _plan_gemm(M=512, N=512, K=k_ok, wb=wb, xb=xb, path=A.PATH_AUTO)
+        assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4 and plan.fp4_exact == 1
+        rc, plan = _plan_gemm(M=512, N=512, K=k_bad, wb=wb, xb=xb, path=A.PATH_AUTO)
+        assert rc == 0 and plan.kernel == A.KERNEL_MFMA_I8 and plan.fp4_exact == 0
+        rc, _ = _plan_gemm(M=512, N=512, K=k_bad, wb=wb, xb=xb, path=A.PATH_MFMA)
+        assert rc == A.EUNSUPPORTED
+        g = A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=512, N=512, K=k_bad, wb=wb, xb=xb, path=A.PATH_MFMA)
+        assert L.apnn_gemm(ctypes.byref(g), None) == A.EUNSUPPORTED
+        rc, plan = _plan_gemm(M=512, N=512, K=k_bad, wb=wb, xb=xb, path=A.PATH_VALU)
+        assert rc == 0 and plan.kernel == A.KERNEL_VALU_TILE
+    # convolution: a 1x1 filter over 2^20 stored channels, w1a4: 2^20 * 15 < 2^24 holds, 9 taps do not
+    geo = dict(batch=64, H=8, Wd=8, COUT=512, stride=1, halo=0, wb=1, xb=4)
+    rc, plan = _plan_conv(cin_pad=2 ** 20, R=1, S=1, pad=0, path=A.PATH_AUTO, **geo)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4
+    rc, plan = _plan_conv(cin_pad=2 ** 18, R=3, S=3, pad=1, path=A.PATH_AUTO, **geo)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_I8 and plan.fp4_exact == 0
+    for pinned in (A.PATH_MFMA, A.PATH_MFMA_PATCH):
+        rc, _ = _plan_conv(cin_pad=2 ** 18, R=3, S=3, pad=1, path=pinned, **geo)
+        assert rc == A.EUNSUPPORTED
+    # wide precisions have no int8 kernel: beyond the bound the VALU path serves them
+    rc, plan = _plan_gemm(M=512, N=512, K=2 ** 17, wb=1, xb=8, path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_VALU_TILE and plan.fp4_exact == 0
+    rc, plan = _plan_gemm(M=512, N=512, K=2 ** 15, wb=1, xb=8, path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4
+
+
+def test_plan_reports_the_dispatchers_choices():
+    """Without a device the dispatcher assumes 256 compute units: the choices for the benchmark shapes."""
+    rc, plan = _plan_gemm(M=64, N=1024, K=1024, wb=1, xb=2, path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_VALU_DIRECT and plan.path == A.PATH_VALU
+    rc, plan = _plan_gemm(M=8192, N=8192, K=8192, wb=1, xb=2, path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4 and (plan.tile_rows, plan.tile_cols) == (256, 128)
+    assert plan.workgroups == 32 * 64
+    rc, plan = _plan_conv(batch=1, H=16, Wd=16, cin_pad=1024, COUT=1024, R=3, S=3, stride=1, pad=1, halo=1, wb=1, xb=2,
+                          path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4 and plan.split_k == 4
+    rc, plan = _plan_conv(batch=64, H=56, Wd=56, cin_pad=64, COUT=64, R=3, S=3, stride=1, pad=1, halo=0, wb=1, xb=2,
+                          path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_PATCH_FP4 and plan.patch_pixels > 0
+    assert A.lib().apnn_gemm_plan(None, ctypes.byref(A.Plan())) == A.ENULL
+    g = A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=64, N=64, K=128, wb=1, xb=2)
+    assert A.lib().apnn_gemm_plan(ctypes.byref(g), None) == A.ENULL
+
+
+def test_patch_capacity_bounds_every_tile():
+    """The patch-resident convolution kernel stages, per work-group, the contiguous range of padded-frame
+    pixels that its tile of consecutive output rows reads; the host sizes that range from a closed-form
+    bound.  Brute force over every tile start of many geometries: the bound is never below the true span
+    (a tile whose span exceeded it would be dropped by the kernel)."""
+    tiles = [(128, 128), (256, 64), (64, 128), (128, 64), (64, 64)]
+    geoms = [  # batch H W R S stride pad pool
+        (3, 16, 16, 3, 3, 1, 1, 0), (2, 56, 56, 3, 3, 1, 1, 0), (5, 7, 7, 3, 3, 1, 1, 0), (4, 14, 14, 3, 3, 2, 1, 0),
+        (3, 28, 28, 1, 1, 2, 0, 0), (2, 13, 11, 5, 5, 1, 2, 0), (2, 12, 20, 3, 3, 1, 1, 1), (3, 8, 8, 5, 3, 1, 1, 2),
+        (9, 5, 6, 3, 3, 1, 1, 0), (2, 30, 9, 3, 1, 1, 0, 0), (7, 6, 6, 3, 3, 1, 1, 1), (2, 24, 24, 5, 5, 2, 2, 1),
+        (70, 3, 3, 3, 3, 1, 1, 0), (1, 40, 6, 1, 5, 1, 2, 0), (6, 10, 10, 3, 3, 1, 0, 1),
+    ]
+    checked = 0
+    for (batch, H, W, R, S, stride, pad, pool) in geoms:
+        PHs, PWs = H + 2 * pad, W + 2 * pad
+        Ho, Wo = (PHs - R) // stride + 1, (PWs - S) // stride + 1
+        if pool and (Ho % 2 or Wo % 2):
+            continue
+        # padded-frame base of every output row, in the kernel's row order
+        bases = []
+        if not pool:
+            for b in range(batch):
+                for oy in range(Ho):
+                    for ox in range(Wo):
+                        bases.append((b * PHs + oy * stride) * PWs + ox * stride)
+        else:
+            for b in range(batch):
+                for py in range(Ho // 2):
+                    for px in range(Wo // 2):
+                        for sub in range(4):
+                            oy, ox = 2 * py + (sub >> 1), 2 * px + (sub & 1)
+                            bases.append((b * PHs + oy * stride) * PWs + ox * stride)
+        for t, (tr, tc) in enumerate(tiles):
+            epi = A.Epilogue()
+            if pool:
+                epi.mode, epi.out_bits, epi.pool = A.EPI_LOWBITS, 2, pool
+            rc, plan = _plan_conv(batch=batch, H=H, Wd=W, cin_pad=64, COUT=64, R=R, S=S, stride=stride, pad=pad, halo=0,
+                                  wb=1, xb=2, epi=epi, path=A.PATH_MFMA_PATCH | ((t + 1) << 8))
+            if rc == A.EUNSUPPORTED:      # patch or filter block does not fit in LDS
+                continue
+            assert rc == 0 and (plan.tile_rows, plan.tile_cols) == (tr, tc)
+            worst = 0
+            for a0 in range(0, len(bases), tr):
+                seg = bases[a0:a0 + tr]
+                worst = max(worst, max(seg) - min(seg) + (R - 1) * PWs + S)
+            assert worst <= plan.patch_pixels <= 1024, (batch, H, W, R, S, stride, pad, pool, t, worst, plan.patch_pixels)
+            checked += 1
+    assert checked >= 40

@@ -79,7 +79,7 @@ def _check_network(G, kind, batch, path, graph):
                 Wt = _download(L, d.weights, d.w_bits * d.out_c * d.R * d.S * cw, np.uint32)
                 thr = _download(L, d.thresholds, d.out_c * nt, np.int32).reshape(d.out_c, nt)
                 acc = O.conv(Wt, X, batch=batch, H=d.in_h, W=d.in_w, cwords=cw, cout=d.out_c, R=d.R, S=d.S,
-                             stride=d.stride, pad=d.pad, halo=0, wb=d.w_bits, xb=d.a_bits, sym_w=1, nthreads=8)
+                             stride=d.stride, pad=d.pad, halo=0, wb=d.w_bits, xb=d.a_bits, sym_w=1, nthreads=16)
                 if d.shortcut_layer >= 0:
                     sd = descs[d.shortcut_layer]
                     srows = batch * sd.out_h * sd.out_w
@@ -113,6 +113,21 @@ def _check_network(G, kind, batch, path, graph):
         return n
     finally:
         L.apnn_net_destroy(net)
+
+
+@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("batch", [8, 64])
+def test_resnet18_benchmark_batches(G, batch, graph):
+    """Batch 8 and 64 (the benchmark's configurations): the library's kernel choice depends on the batch
+    (tile shapes, split-K, the patch-resident kernel), so the small-batch test does not cover them."""
+    assert _check_network(G, G.A.NET_RESNET18, batch, 0, graph=graph) == 21
+
+
+@pytest.mark.parametrize("kind,layers", [("alexnet", 8), ("vgg", 13)])
+def test_alexnet_and_vgg_batch8(G, kind, layers):
+    net = G.A.NET_ALEXNET if kind == "alexnet" else G.A.NET_VGG
+    assert _check_network(G, net, 8, 0, graph=False) == layers
+    assert _check_network(G, net, 8, 0, graph=True) == layers
 
 
 @pytest.mark.parametrize("path", [0, 1, 2])

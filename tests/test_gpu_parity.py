@@ -50,12 +50,16 @@ def test_gemm_named_entry_golden(G, wb, xb):
     assert np.array_equal(gotp, O.lowbits_pack(_golden()["gemm_" + name], M, N, xb))
 
 
-PATHS = [1, 2, 3]   # APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8 (GEMM entry points only)
-CONV_PATHS = [1, 2, 4]   # 4 = APNN_PATH_MFMA_PATCH (input patch resident in LDS)
+# 0 = APNN_PATH_AUTO (the library's own choice: what the named entry points, the networks and the
+# benchmark run), APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8
+PATHS = [0, 1, 2, 3]
+CONV_PATHS = [0, 1, 2, 3, 4]   # 4 = APNN_PATH_MFMA_PATCH (input patch resident in LDS)
 # (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
-# int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128
+# int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128; int8 convolution
+# 128x128, 64x64, 128x64, 32x32 split-K, 128x256
 GEMM_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)]
-CONV_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)] + [(4, t) for t in range(5)]
+CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
+              [(4, t) for t in range(5)])
 GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
 CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
 
@@ -180,6 +184,32 @@ def test_conv3x3_16x16_sweep(G, wb, xb, C, batch, path):
     assert np.array_equal(got, O.conv(Wt, X, cwords=C // 32, nthreads=8, **kw))
 
 
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("batch", [1, 16])
+@pytest.mark.parametrize("C", [128, 256, 384, 512, 640, 768, 896, 1024])
+def test_conv3x3_16x16_benchmark_shapes_auto(G, wb, xb, C, batch):
+    """Every shape of the 16x16 benchmark family on the library's own kernel choice: int32 output, then
+    the fused BN-threshold requantize to a bits with thresholds drawn as sorted uniform integers in
+    [0, 9*Cin*(2^a-1)(2^w-1)/2] per channel, packed for the next layer."""
+    rng = np.random.default_rng(3300 + C + batch + wb * 3 + xb)
+    H = Wd = 16
+    X = O.random_planes(rng, xb, batch * (H + 2) * (Wd + 2), C // 32)
+    Wt = O.random_planes(rng, wb, C * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=1, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, nthreads=16, **kw)
+    got = G.run_conv(Wt, X, cin_pad=C, path=0, **kw).reshape(acc.shape)
+    assert np.array_equal(got, acc)
+    hi = 9 * C * (2 ** xb - 1) * (2 ** wb - 1) // 2
+    thr = np.sort(rng.integers(0, hi + 1, size=(C, 2 ** xb - 1)), axis=1).astype(np.int32)
+    d_thr = G.to_dev(thr)
+    rows = batch * H * Wd
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=xb, thr=d_thr)
+    gotq = G.run_conv(Wt, X, cin_pad=C, epi=epi, path=0, **kw).view(np.uint32).reshape(xb, rows, C // 32)
+    q = O.bn_quantize(acc.reshape(rows, C), None, thr, None, xb)
+    assert 0 < q.mean() < 2 ** xb - 1
+    assert np.array_equal(gotq, O.lowbits_pack(q, rows, C, xb))
+
+
 GEOMS = [  # batch H W cin_pad cout R stride pad halo
     (2, 14, 14, 128, 96, 3, 1, 1, 0),     # predicated halo, cout not a tile multiple
     (3, 28, 28, 64, 128, 3, 2, 1, 0),     # ResNet stride-2 3x3 on 64 stored channels (64-bit loads)
@@ -302,6 +332,27 @@ def test_gemm_2048_sampled_and_closed_form(G, wb, xb, path):
     ones_w = np.full_like(W, 0xFFFFFFFF)
     ones_x = np.full_like(X, 0xFFFFFFFF)
     assert np.all(G.run_gemm(ones_w, ones_x, M, N, K, wb, xb, path=path) == K * (2 ** wb - 1) * (2 ** xb - 1))
+
+
+@pytest.mark.parametrize("wb,xb", COMBOS)
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_gemm_large_auto_sampled_linearity_closed_form(G, wb, xb, n):
+    """M = N = K = 4096 / 8192 on the library's own kernel choice.  The oracle is too slow for 7e10 /
+    5e11 outputs' worth of work, so: rows sampled at random against the oracle, every column sum against
+    the linear form (each output element takes part), and the all-ones closed form K(2^w-1)(2^a-1)."""
+    rng = np.random.default_rng(8800 + n + wb * 5 + xb)
+    M = N = K = n
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, path=0).reshape(M, N)
+    rows = sorted(set([0, M - 1] + [int(v) for v in rng.choice(M, 22, replace=False)]))
+    for m in rows:
+        assert np.array_equal(got[m], O.gemm_rows(W, X, M, N, K, wb, xb, m, m + 1, nthreads=16)[0]), m
+    assert np.array_equal(got.sum(0, dtype=np.int64), O.gemm_column_sums(W, X))
+    del got
+    W[:] = 0xFFFFFFFF
+    X[:] = 0xFFFFFFFF
+    assert np.all(G.run_gemm(W, X, M, N, K, wb, xb, path=0) == K * (2 ** wb - 1) * (2 ** xb - 1))
 
 
 # ---- layers on either side of the low-bit path ---------------------------------------------------
@@ -569,7 +620,65 @@ def test_gemm_named_entry_more_precisions(G, wb, xb):
     assert fn(G.ptr(dW), G.ptr(dX), G.ptr(out), M, N, K, wb + 1, xb, None) == G.A.EINVAL
 
 
+@pytest.mark.parametrize("wb,xb", [(4, 4), (1, 8), (2, 8)])
+@pytest.mark.parametrize("tile", [None, 1, 2, 4])
+@pytest.mark.parametrize("sym", [0, 1])
+def test_wide_precisions_on_the_matrix_cores(G, wb, xb, tile, sym):
+    """w4a4 / w1a8 / w2a8 as FP4 digit pairs (2 x 2, 1 x 4, 1 x 4 MFMAs per block and k-step, weighted by
+    the block scale): GEMM and convolution, int32 and quantized packed output, every tile that is built."""
+    rng = np.random.default_rng(5300 + 100 * wb + 10 * xb + (tile or 0) + sym)
+    M, N, K = 150, 200, 1152
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, wb, xb, sym_w=sym, nthreads=8)
+    if not sym:
+        assert np.array_equal(acc, O.unpack_planes_lsb(W) @ O.unpack_planes_lsb(X).T)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=2, tile=tile).reshape(M, N)
+    assert np.array_equal(got, acc)
+    batch, H, Wd, C, cout = 2, 9, 10, 128, 96
+    Xc = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wc = O.random_planes(rng, wb, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    cacc = O.conv(Wc, Xc, cwords=C // 32, sym_w=sym, nthreads=8, **kw)
+    assert np.array_equal(G.run_conv(Wc, Xc, cin_pad=C, sym=sym, path=2, tile=tile, **kw).reshape(cacc.shape), cacc)
+    for ob in (2, 4, 8):
+        span = int(np.abs(cacc).max())
+        thr = np.sort(rng.integers(-span if sym else 0, span, size=(cout, 2 ** ob - 1)), axis=1).astype(np.int32)
+        d_thr = G.to_dev(thr)
+        epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr)
+        rows = batch * H * Wd
+        gotq = G.run_conv(Wc, Xc, cin_pad=C, sym=sym, epi=epi, path=2, tile=tile, **kw).view(np.uint32).reshape(ob, rows, cout // 32)
+        assert np.array_equal(gotq, O.lowbits_pack(O.bn_quantize(cacc.reshape(rows, cout), None, thr, None, ob), rows, cout, ob))
+    if tile is None:     # 64 stored channels: 64-bit loads, where only the 64x64 tile is built
+        Xn = O.random_planes(rng, xb, batch * H * Wd, 2)
+        Wn = O.random_planes(rng, wb, cout * 9, 2)
+        nacc = O.conv(Wn, Xn, cwords=2, sym_w=sym, **kw)
+        assert np.array_equal(G.run_conv(Wn, Xn, cin_pad=64, sym=sym, path=2, **kw).reshape(nacc.shape), nacc)
+
+
+def test_fp4_guard_falls_back_to_int32_accumulation(G):
+    """K * 15 >= 2^24 for w1a4: all-ones operands make every output K * 15, which fp32 cannot hold.  The
+    library's own choice must still be exact (int8 core); the FP4 path refuses."""
+    M = N = 288
+    K = 1179648
+    W = np.full((1, M, K // 32), 0xFFFFFFFF, np.uint32)
+    X = np.full((4, N, K // 32), 0xFFFFFFFF, np.uint32)
+    assert K * 15 >= 2 ** 24
+    plan = G.A.Plan()
+    d = G.A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=M, N=N, K=K, wb=1, xb=4)
+    assert G.A.lib().apnn_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.kernel == G.A.KERNEL_MFMA_I8
+    assert np.all(G.run_gemm(W, X, M, N, K, 1, 4, path=0) == K * 15)
+    with pytest.raises(G.A.ApnnError, match="EUNSUPPORTED"):
+        G.run_gemm(W, X, M, N, K, 1, 4, path=2)
+    # random weights against one all-ones activation row: popcounts of the weight rows times 15
+    Wr = O.random_planes(np.random.default_rng(5), 1, M, K // 32)
+    got = G.run_gemm(Wr, X, M, N, K, 1, 4, path=0).reshape(M, N)
+    pop = np.array([int(np.unpackbits(Wr[0, m].view(np.uint8)).sum()) for m in range(M)])
+    assert np.array_equal(got, np.repeat((15 * pop)[:, None], N, axis=1))
+
+
 @pytest.mark.parametrize("name,wb,xb,pack", [("apconv_w1a5", 1, 5, False), ("apconv_w2a6", 2, 6, False),
+                                             ("apconv_w1a8", 1, 8, False), ("apconv_w2a8", 2, 8, False),
                                              ("APConv_w2a8_pack", 2, 8, True)])
 def test_conv_named_entry_more_precisions(G, name, wb, xb, pack):
     rng = np.random.default_rng(5100 + 10 * wb + xb)
@@ -587,6 +696,12 @@ def test_conv_named_entry_more_precisions(G, name, wb, xb, pack):
     if pack:
         expect = O.lowbits_pack(acc.reshape(-1, cout), H * Wd, cout, xb)
         assert np.array_equal(G.to_host(out, np.uint32).reshape(expect.shape), expect)
+        # 2x2 average pool (C integer division) before the low bits: APConv_w2a8_pack_pool
+        outq = G.dev_empty_i32(xb * (H // 2) * (Wd // 2) * cout // 32, fill=-7)
+        G.A.check(getattr(G.A.lib(), name + "_pool")(G.ptr(dW), G.ptr(dX), G.ptr(outq), H, Wd, C, cout, None), name)
+        pooled = O.avgpool2x2(acc)[0]
+        expq = O.lowbits_pack(pooled, (H // 2) * (Wd // 2), cout, xb)
+        assert np.array_equal(G.to_host(outq, np.uint32).reshape(expq.shape), expq)
     else:
         assert np.array_equal(G.to_host(out).reshape(acc.shape), acc)
 

@@ -6,6 +6,18 @@ import pytest
 import oracle_lib as O
 
 
+def _golden():
+    import os
+    return np.load(os.path.join(O.GOLDEN_DIR, "golden_outputs.npz"), allow_pickle=False)
+
+
+def test_fnv1a64_is_the_published_function():
+    """Published FNV-1a-64 test vectors: the empty string is the offset basis, "a" and "foobar"."""
+    assert O.fnv1a64(np.zeros(0, np.uint8)) == 0xcbf29ce484222325
+    assert O.fnv1a64(np.frombuffer(b"a", np.uint8)) == 0xaf63dc4c8601ec8c
+    assert O.fnv1a64(np.frombuffer(b"foobar", np.uint8)) == 0x85944171f73967e8
+
+
 def _gemm_inputs_from_stream(M, N, K, wb, xb):
     s = O.golden_stream()
     nw, nx = wb * M * K // 32, xb * N * K // 32
@@ -32,6 +44,8 @@ def test_gemm_known_answers(name):
         flat = D.ravel()
         assert (int(flat[0]), int(flat[1]), int(flat[-1])) == (c["c0"], c["c1"], c["clast"])
         assert int(flat.astype(np.int64).sum()) == c["sum"]
+        assert "%016x" % O.fnv1a64(D.astype("<i4")) == c["fnv"]
+    assert "%016x" % O.fnv1a64(_golden()["gemm_" + name].astype("<i4")) == c["fnv"]
 
 
 @pytest.mark.parametrize("name", ["w1a2", "w1a3", "w1a4", "w2a2"])
@@ -48,8 +62,13 @@ def test_conv_known_answers(name):
         flat = D.ravel()
         assert (int(flat[0]), int(flat[1])) == (c["c0"], c["c1"])
         assert int(flat.astype(np.int64).sum()) == c["sum"]
+        assert "%016x" % O.fnv1a64(D.astype("<i4")) == c["fnv"]
     packed = O.lowbits_pack(lit, H * Wd, COUT, c["xb"])
     assert "%08x" % int(packed.ravel()[0]) == c["pack0"]
+    assert "%016x" % O.fnv1a64(packed.astype("<u4")) == c["pack_fnv"]
+    gold = _golden()
+    assert "%016x" % O.fnv1a64(gold["conv_" + name].astype("<i4")) == c["fnv"]
+    assert "%016x" % O.fnv1a64(gold["conv_pack_" + name].astype("<u4")) == c["pack_fnv"]
 
 
 def test_plane_product_kat():
