@@ -61,7 +61,8 @@ _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2", "apco
 DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
                                                 "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
                                                 "apnn_conv_i8_bn_pack", "apnn_pool_planes", "apnn_quantize_pack", "apnn_fold_bn", "apnn_conv_pair",
-                                                "apnn_gemm_plan", "apnn_conv_plan",
+                                                "apnn_gemm_plan", "apnn_conv_plan", "apnn_quantize_pack_u8", "apnn_binarize_pack",
+                                                "apnn_residual_prepare",
                                                 "apnn_device_cus", "apnn_version"]
 
 
@@ -133,6 +134,12 @@ def lib():
         L.apnn_fc_i8.restype = _ci
         L.apnn_quantize_pack.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, ctypes.c_float, ctypes.c_float, _vp]
         L.apnn_quantize_pack.restype = _ci
+        L.apnn_quantize_pack_u8.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]
+        L.apnn_quantize_pack_u8.restype = _ci
+        L.apnn_binarize_pack.argtypes = [_vp, _vp, _ci, _ci, _ci, _vp]
+        L.apnn_binarize_pack.restype = _ci
+        L.apnn_residual_prepare.argtypes = [_vp, _vp] + [_ci] * 7 + [_vp]
+        L.apnn_residual_prepare.restype = _ci
         L.apnn_fold_bn.argtypes = [_vp] * 4 + [ctypes.c_float] * 3 + [_ci, _ci, _vp, _vp]
         L.apnn_fold_bn.restype = _ci
         L.apnn_device_cus.argtypes = []

@@ -122,6 +122,7 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   if (i8) return nullptr;
   if (xb == 8 && wb == 1) return apnn::mfma4_conv_8_1_x;
   if (xb == 8 && wb == 2) return apnn::mfma4_conv_8_2_x;
+  if (xb == 4 && wb == 4) return apnn::mfma4_conv_4_4_x;
   return nullptr;
 }
 
@@ -680,6 +681,29 @@ int apnn_quantize_pack(const float *values, uint32_t *planes, int rows, int C, i
     return APNN_EINVAL;
   return (int)apnn::launch_quantize_pack(values, planes, rows, C, cpad, bits, min_v, max_v,
                                          static_cast<hipStream_t>(s));
+}
+
+int apnn_quantize_pack_u8(const uint8_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                          apnn_stream_t s) {
+  if (values == nullptr || planes == nullptr) return APNN_ENULL;
+  if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 8) return APNN_EINVAL;
+  return (int)apnn::launch_quantize_pack_u8(values, planes, rows, C, cpad, bits, static_cast<hipStream_t>(s));
+}
+
+int apnn_binarize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, apnn_stream_t s) {
+  if (values == nullptr || planes == nullptr) return APNN_ENULL;
+  if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0) return APNN_EINVAL;
+  return (int)apnn::launch_binarize_pack(values, planes, rows, C, cpad, static_cast<hipStream_t>(s));
+}
+
+int apnn_residual_prepare(const int32_t *in, int32_t *out, int B, int Ho, int Wo, int in_pitch, int channels,
+                          int out_channels, int pool, apnn_stream_t s) {
+  if (in == nullptr || out == nullptr) return APNN_ENULL;
+  if (B <= 0 || Ho <= 0 || Wo <= 0 || out_channels <= 0 || channels < 0 || channels > out_channels ||
+      in_pitch < channels || (pool != 0 && pool != 1))
+    return APNN_EINVAL;
+  return (int)apnn::launch_residual_prepare(in, out, B, Ho, Wo, in_pitch, channels, out_channels, pool,
+                                            static_cast<hipStream_t>(s));
 }
 
 int apnn_fold_bn(const float *gamma, const float *beta, const float *mean, const float *var, float eps,

@@ -41,8 +41,11 @@ int timed_loop(F &&launch, int warmup, int iters, hipStream_t stream, float *eve
 
 // Same measurement with the launches replayed from a HIP graph: `batch` launches are captured once
 // (on a stream of its own, default priority) and the graph is launched ceil(n / batch) times, the last
-// time through a second graph holding the remainder, so exactly `warmup` + `iters` kernels run.  The
-// host then issues one graph launch per `batch` kernels instead of one call per kernel.
+// time through a second graph holding the remainder, so exactly `iters` kernels run in the timed region.
+// The host then issues one graph launch per `batch` kernels instead of one call per kernel.  Every
+// executable graph the timed region uses is launched once, untimed, beforehand (the first launch of a
+// graph pays for its upload to the device: a timed region of one or two graph launches would otherwise
+// measure that), so at least `warmup` untimed kernels run, rounded up to whole graphs.
 template <class F>
 int timed_graph_loop(F &&launch_on, int warmup, int iters, int batch, float *event_ms, double *wall_ms) {
   if (batch < 1) batch = 1;
@@ -83,6 +86,8 @@ int timed_graph_loop(F &&launch_on, int warmup, int iters, int batch, float *eve
   if (rc == 0 && (err = hipEventCreate(&e0)) != hipSuccess) rc = (int)err;
   if (rc == 0 && (err = hipEventCreate(&e1)) != hipSuccess) rc = (int)err;
   if (rc == 0) rc = replay(warmup, rest_w);
+  if (rc == 0 && warmup < batch && iters >= batch && (err = hipGraphLaunch(full, cs)) != hipSuccess) rc = (int)err;
+  if (rc == 0 && rest_i != nullptr && (err = hipGraphLaunch(rest_i, cs)) != hipSuccess) rc = (int)err;
   if (rc == 0 && (err = hipStreamSynchronize(cs)) != hipSuccess) rc = (int)err;
   if (rc == 0) {
     const auto t0 = std::chrono::steady_clock::now();

@@ -37,6 +37,7 @@ APNN_DECL_MFMA4(gemm, 1, 8)
 APNN_DECL_MFMA4(gemm, 2, 8)
 APNN_DECL_MFMA4(conv, 8, 1)
 APNN_DECL_MFMA4(conv, 8, 2)
+APNN_DECL_MFMA4(conv, 4, 4)
 APNN_DECL_MFMA4(gemm, 1, 2)
 APNN_DECL_MFMA4(gemm, 1, 3)
 APNN_DECL_MFMA4(gemm, 1, 4)
@@ -100,6 +101,12 @@ hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, 
 
 hipError_t launch_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
                                 float max_v, hipStream_t s);
+
+hipError_t launch_quantize_pack_u8(const uint8_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                                   hipStream_t s);
+hipError_t launch_binarize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, hipStream_t s);
+hipError_t launch_residual_prepare(const int32_t *in, int32_t *out, int B, int Ho, int Wo, int in_pitch, int channels,
+                                   int out_channels, int pool, hipStream_t s);
 
 // nn_kernels.hip
 hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *thr, uint8_t *codes, int32_t *acc_out,

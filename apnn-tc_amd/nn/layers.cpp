@@ -76,16 +76,79 @@ static std::vector<T> download(const void *dev, size_t count) {
   return host;
 }
 
+// ---- In128LayerParam / ImageQuantLayerParam -----------------------------------------------------------
+
+static void clear_desc(apnn_layer_desc *d, const std::string &name, int kind, int batch) {
+  std::memset(d, 0, sizeof(*d));
+  copy_name(d->name, name);
+  d->kind = kind;
+  d->batch = batch;
+  d->shortcut_layer = -1;
+  d->residual_layer = -1;
+  d->global_pool_shift = -1;
+}
+
+In128LayerParam::In128LayerParam(const char *name_, int input_height_, int input_width_)
+    : name(name_), input_height(input_height_), input_width(input_width_), output_height(input_height_),
+      output_width(input_width_), out_cpad(pad_to(input_width_, 32)) {}
+
+int In128LayerParam::initialize(const float *input_gpu_) {
+  if (output_gpu.allocate((size_t)output_height * (out_cpad / 32) * 4) != hipSuccess) return 1;
+  input_gpu = input_gpu_;
+  return 0;
+}
+
+int In128LayerParam::forward(hipStream_t stream) {
+  return apnn_binarize_pack(input_gpu, output_gpu.as<uint32_t>(), input_height, input_width, out_cpad, stream);
+}
+
+void In128LayerParam::describe(apnn_layer_desc *d) const {
+  clear_desc(d, name, APNN_LAYER_IMAGE_QUANT, input_height);
+  d->in_h = 1, d->in_w = 1, d->in_c = input_width, d->in_cpad = input_width;
+  d->out_h = 1, d->out_w = 1, d->out_c = input_width, d->out_cpad = out_cpad;
+  d->a_bits = 32, d->out_bits = 1;
+  d->input = input_gpu, d->output = output_gpu.get();
+}
+
+ImageQuantLayerParam::ImageQuantLayerParam(const char *name_, int batch_, int image_height_, int image_width_,
+                                           int image_channel_, int bit_)
+    : name(name_), batch(batch_), image_height(image_height_), image_width(image_width_),
+      image_channel(image_channel_), bit(bit_), out_cpad(pad_to(image_channel_, 32)) {}
+
+int ImageQuantLayerParam::initialize(const uint8_t *images_gpu) {
+  if (output_gpu.allocate((size_t)bit * batch * image_height * image_width * (out_cpad / 32) * 4) != hipSuccess) return 1;
+  input_gpu = images_gpu;
+  return 0;
+}
+
+int ImageQuantLayerParam::forward(hipStream_t stream) {
+  return apnn_quantize_pack_u8(input_gpu, output_gpu.as<uint32_t>(), batch * image_height * image_width, image_channel,
+                               out_cpad, bit, stream);
+}
+
+void ImageQuantLayerParam::describe(apnn_layer_desc *d) const {
+  clear_desc(d, name, APNN_LAYER_IMAGE_QUANT, batch);
+  d->in_h = image_height, d->in_w = image_width, d->in_c = image_channel, d->in_cpad = image_channel;
+  d->out_h = image_height, d->out_w = image_width, d->out_c = image_channel, d->out_cpad = out_cpad;
+  d->a_bits = 8, d->out_bits = bit;
+  d->input = input_gpu, d->output = output_gpu.get();
+}
+
 // ---- InConv128LayerParam ---------------------------------------------------------------------------
 
 InConv128LayerParam::InConv128LayerParam(const char *name_, int input_height_, int input_width_, int filter_height_,
                                          int filter_width_, int input_channels_, int output_channels_, int batch_,
-                                         int stride_height, int /*stride_width*/, bool padding, int pool_height,
-                                         int /*pool_width*/, int pool_stride_, int pool_pad_, int a_bit_)
+                                         int stride_height, int stride_width, bool padding, int pool_height,
+                                         int pool_width, bool save_residual_, int pool_stride_, int pool_pad_,
+                                         int a_bit_)
     : name(name_), input_height(input_height_), input_width(input_width_), filter_height(filter_height_),
       filter_width(filter_width_), input_channels(input_channels_), output_channels(output_channels_), batch(batch_),
       stride(stride_height), pad(padding ? (filter_height_ - 1) / 2 : 0), pool(pool_height),
-      pool_stride(pool_stride_ > 0 ? pool_stride_ : pool_height), pool_pad(pool_pad_), a_bit(a_bit_) {
+      pool_stride(pool_stride_ > 0 ? pool_stride_ : pool_height), pool_pad(pool_pad_), a_bit(a_bit_),
+      save_residual(save_residual_) {
+  if (stride_width != stride_height || pool_width != pool_height || pool_height < 1 ||
+      (padding && ((filter_height_ | filter_width_) & 1) == 0))
+    status = APNN_EUNSUPPORTED;
   conv_height = (input_height + 2 * pad - filter_height) / stride + 1;
   conv_width = (input_width + 2 * pad - filter_width) / stride + 1;
   output_height = (conv_height + 2 * pool_pad - pool) / pool_stride + 1;
@@ -94,6 +157,7 @@ InConv128LayerParam::InConv128LayerParam(const char *name_, int input_height_, i
 }
 
 int InConv128LayerParam::initialize(Rng &rng, const uint8_t *images_gpu) {
+  if (status != 0) return status;
   const size_t nw = (size_t)output_channels * filter_height * filter_width * input_channels;
   std::vector<int8_t> w(nw);
   for (auto &v : w) v = (int8_t)((int)rng.below(255) - 127);
@@ -102,10 +166,14 @@ int InConv128LayerParam::initialize(Rng &rng, const uint8_t *images_gpu) {
   const double sigma = std::sqrt((double)filter_height * filter_width * input_channels * 5461.0 * 5376.0);
   const std::vector<int32_t> thr = random_thresholds(rng, output_channels, a_bit, 0.0, sigma);
   if (bn_gpu.upload(thr.data(), thr.size() * sizeof(int32_t)) != hipSuccess) return 1;
-  // un-pooled packed codes of the convolution (skipped when there is no pooling stage)
-  if (pool > 1 &&
-      codes_gpu.allocate((size_t)a_bit * batch * conv_height * conv_width * (out_cpad / 32) * 4) != hipSuccess)
-    return 1;
+  const size_t conv_px = (size_t)batch * conv_height * conv_width;
+  if (save_residual) {
+    // the kernel that also writes the int32 sums produces byte codes; they are pooled and packed after it
+    if (codes_gpu.allocate(conv_px * output_channels) != hipSuccess) return 1;
+    if (output_residual_gpu.allocate(conv_px * output_channels * sizeof(int32_t)) != hipSuccess) return 1;
+  } else if (pool > 1 && codes_gpu.allocate((size_t)a_bit * conv_px * (out_cpad / 32) * 4) != hipSuccess) {
+    return 1;  // un-pooled packed codes of the convolution (skipped when there is no pooling stage)
+  }
   if (output_gpu.allocate((size_t)a_bit * batch * output_height * output_width * (out_cpad / 32) * 4) != hipSuccess)
     return 1;
   input_gpu = images_gpu;
@@ -113,6 +181,15 @@ int InConv128LayerParam::initialize(Rng &rng, const uint8_t *images_gpu) {
 }
 
 int InConv128LayerParam::forward(hipStream_t stream) {
+  if (save_residual) {
+    int rc = apnn_conv_i8_bn(reinterpret_cast<const int8_t *>(input_gpu), filter_gpu.as<int8_t>(), bn_gpu.as<int32_t>(),
+                             codes_gpu.as<uint8_t>(), output_residual_gpu.as<int32_t>(), batch, input_height,
+                             input_width, input_channels, output_channels, filter_height, filter_width, stride, pad,
+                             a_bit, 128, stream);
+    if (rc != 0) return rc;
+    return apnn_pool_pack(codes_gpu.as<uint8_t>(), output_gpu.as<uint32_t>(), batch, conv_height, conv_width,
+                          output_channels, out_cpad, a_bit, pool, pool_stride, pool_pad, stream);
+  }
   uint32_t *conv_out = pool > 1 ? codes_gpu.as<uint32_t>() : output_gpu.as<uint32_t>();
   int rc = apnn_conv_i8_bn_pack(reinterpret_cast<const int8_t *>(input_gpu), filter_gpu.as<int8_t>(),
                                 bn_gpu.as<int32_t>(), conv_out, batch, input_height, input_width, input_channels,
@@ -123,17 +200,14 @@ int InConv128LayerParam::forward(hipStream_t stream) {
 }
 
 void InConv128LayerParam::describe(apnn_layer_desc *d) const {
-  std::memset(d, 0, sizeof(*d));
-  copy_name(d->name, name);
-  d->kind = APNN_LAYER_INCONV_I8;
-  d->batch = batch;
+  clear_desc(d, name, APNN_LAYER_INCONV_I8, batch);
   d->in_h = input_height, d->in_w = input_width, d->in_c = input_channels, d->in_cpad = input_channels;
   d->out_h = output_height, d->out_w = output_width, d->out_c = output_channels, d->out_cpad = out_cpad;
   d->R = filter_height, d->S = filter_width, d->stride = stride, d->pad = pad;
   d->pool_win = pool > 1 ? pool : 0, d->pool_stride = pool_stride, d->pool_pad = pool_pad;
   d->a_bits = 8, d->w_bits = 8, d->out_bits = a_bit;
-  d->shortcut_layer = -1;
-  d->global_pool_shift = -1;
+  d->save_residual = save_residual ? 1 : 0;
+  d->residual_out = output_residual_gpu.get();
   d->input = input_gpu, d->weights = filter_gpu.get(), d->thresholds = bn_gpu.get(), d->output = output_gpu.get();
 }
 
@@ -145,14 +219,21 @@ std::vector<uint32_t> InConv128LayerParam::download_output() const {
 
 Conv128LayerParam::Conv128LayerParam(const char *name_, int input_height_, int input_width_, int filter_height_,
                                      int filter_width_, int input_channels_, int output_channels_, int batch_,
-                                     int stride_height, int /*stride_width*/, bool padding, int pool_height,
-                                     int /*pool_width*/, bool /*ahead_fc*/, bool /*save_residual*/,
-                                     bool inject_residual_, int /*residual_channels*/, bool /*residual_pool*/,
-                                     int a_bit_, int w_bit_)
+                                     int stride_height, int stride_width, bool padding, int pool_height,
+                                     int pool_width, bool ahead_fc_, bool save_residual_, bool inject_residual_,
+                                     int residual_channels_, bool residual_pool_, int a_bit_, int w_bit_)
     : name(name_), input_height(input_height_), input_width(input_width_), filter_height(filter_height_),
       filter_width(filter_width_), input_channels(input_channels_), output_channels(output_channels_), batch(batch_),
       stride(stride_height), pad(padding ? (filter_height_ - 1) / 2 : 0), pool(pool_height), a_bit(a_bit_),
-      w_bit(w_bit_), inject_residual(inject_residual_) {
+      w_bit(w_bit_), ahead_fc(ahead_fc_), save_residual(save_residual_), inject_residual(inject_residual_),
+      residual_pool(residual_pool_), residual_channels(residual_channels_) {
+  // what the kernels behind this class cannot do is refused by initialize(), not dropped: anisotropic
+  // stride / pooling, pooling windows other than 2x2, "same" padding of an even filter, and the int32
+  // residual path together with pooling (the epilogue pools before it could add or save)
+  if (stride_width != stride_height || pool_width != pool_height || (pool_height != 1 && pool_height != 2) ||
+      (padding && ((filter_height_ | filter_width_) & 1) == 0) || filter_height_ != filter_width_ ||
+      ((save_residual_ || inject_residual_) && pool_height != 1) || (inject_residual_ && residual_channels_ <= 0))
+    status = APNN_EUNSUPPORTED;
   // output-size rule of param.h:915-924 for symmetric padding: ceil(in/stride) when padded
   conv_height = (input_height + 2 * pad - filter_height) / stride + 1;
   conv_width = (input_width + 2 * pad - filter_width) / stride + 1;
@@ -162,22 +243,36 @@ Conv128LayerParam::Conv128LayerParam(const char *name_, int input_height_, int i
   out_cpad = pad_to(output_channels, 32);
 }
 
-int Conv128LayerParam::initialize(Rng &rng, const uint32_t *prev_layer_gpu, const uint32_t *input_residual_gpu_,
-                                  int residual_scale_, int path_) {
+int Conv128LayerParam::initialize(Rng &rng, const uint32_t *prev_layer_gpu, const int32_t *input_residual_gpu_,
+                                  int path_, int input_residual_pitch, int residual_layer_) {
+  if (status != 0) return status;
+  if (inject_residual && packed_shortcut_gpu != nullptr) return APNN_EUNSUPPORTED;  // one shortcut form per layer
   int rc = random_planes_gpu(rng, filter_gpu, output_channels * filter_height * filter_width, input_channels, in_cpad,
                              w_bit);
   if (rc != 0) return rc;
-  residual_scale = inject_residual ? residual_scale_ : 0;
   const double amax = (double)((1 << a_bit) - 1), wmax = (double)((1 << w_bit) - 1);
   // codes uniform in 0..amax: E[x^2] = amax(2 amax + 1)/6; symmetric weights uniform in {-wmax..wmax step 2}
   const double ex2 = amax * (2 * amax + 1) / 6.0, ew2 = (wmax * wmax + 2 * wmax) / 3.0;
   const double sigma = std::sqrt((double)filter_height * filter_width * input_channels * ex2 * ew2);
-  const double center = residual_scale * amax / 2.0;
+  const double center = packed_shortcut_gpu != nullptr ? residual_scale * amax / 2.0 : 0.0;
   const std::vector<int32_t> thr = random_thresholds(rng, output_channels, a_bit, center, sigma);
   if (bn_gpu.upload(thr.data(), thr.size() * sizeof(int32_t)) != hipSuccess) return 1;
   if (output_gpu.allocate((size_t)output_bit_words() * 4) != hipSuccess) return 1;
+  if (save_residual && output_residual_gpu.allocate((size_t)residual_words() * sizeof(int32_t)) != hipSuccess) return 1;
   input_gpu = prev_layer_gpu;
-  input_residual_gpu = inject_residual ? input_residual_gpu_ : nullptr;
+  if (inject_residual) {
+    if (input_residual_gpu_ == nullptr) return APNN_ENULL;
+    input_residual_gpu = input_residual_gpu_;
+    residual_layer = residual_layer_;
+    // channels that receive the residual: below residual_channels, and no more than the map holds (the
+    // reference reads zero padding beyond the source layer's channels, kernel.cuh:779-817)
+    residual_pitch = input_residual_pitch > 0 ? input_residual_pitch : std::min(residual_channels, output_channels);
+    residual_used = std::min(std::min(residual_channels, output_channels), residual_pitch);
+    // a map that is not already [rows][output_channels] is brought to that shape before the convolution
+    if ((residual_pool || residual_used != output_channels || residual_pitch != output_channels) &&
+        residual_tmp_gpu.allocate((size_t)residual_words() * sizeof(int32_t)) != hipSuccess)
+      return 1;
+  }
   path = path_;
   return 0;
 }
@@ -204,14 +299,24 @@ static apnn_conv_desc conv_desc_of(const Conv128LayerParam *p) {
   d.epi.out_bits = p->a_bit;
   d.epi.pool = p->pool == 2 ? APNN_POOL_MAX2X2 : APNN_POOL_NONE;
   d.epi.thresholds = p->bn_gpu.as<int32_t>();
-  d.epi.residual_planes = p->input_residual_gpu;
+  d.epi.residual_planes = p->packed_shortcut_gpu;
   d.epi.residual_bits = p->a_bit;
   d.epi.residual_scale = p->residual_scale;
+  if (p->inject_residual)
+    d.epi.residual = p->residual_tmp_gpu.get() != nullptr ? p->residual_tmp_gpu.as<int32_t>() : p->input_residual_gpu;
+  if (p->save_residual) d.epi.save_acc = p->output_residual_gpu.as<int32_t>();
   d.path = p->path;
   return d;
 }
 
 int Conv_new_global(Conv128LayerParam *p, hipStream_t stream) {
+  if (p->inject_residual && p->residual_tmp_gpu.get() != nullptr) {
+    const int rc = apnn_residual_prepare(p->input_residual_gpu, p->residual_tmp_gpu.as<int32_t>(), p->batch,
+                                         p->conv_height, p->conv_width, p->residual_pitch, p->residual_used,
+                                         p->output_channels,
+                                         p->residual_pool ? 1 : 0, stream);
+    if (rc != 0) return rc;
+  }
   const apnn_conv_desc d = conv_desc_of(p);
   return apnn_conv(&d, stream);
 }
@@ -224,10 +329,7 @@ int Conv_pair_global(Conv128LayerParam *main_branch, Conv128LayerParam *shortcut
 int Conv128LayerParam::forward(hipStream_t stream) { return Conv_new_global(this, stream); }
 
 void Conv128LayerParam::describe(apnn_layer_desc *d) const {
-  std::memset(d, 0, sizeof(*d));
-  copy_name(d->name, name);
-  d->kind = APNN_LAYER_CONV;
-  d->batch = batch;
+  clear_desc(d, name, APNN_LAYER_CONV, batch);
   d->in_h = input_height, d->in_w = input_width, d->in_c = input_channels, d->in_cpad = in_cpad;
   d->out_h = output_height, d->out_w = output_width, d->out_c = output_channels, d->out_cpad = out_cpad;
   d->R = filter_height, d->S = filter_width, d->stride = stride, d->pad = pad;
@@ -235,7 +337,14 @@ void Conv128LayerParam::describe(apnn_layer_desc *d) const {
   d->a_bits = a_bit, d->w_bits = w_bit, d->out_bits = a_bit;
   d->shortcut_layer = shortcut_layer;
   d->shortcut_scale = residual_scale;
-  d->global_pool_shift = -1;
+  if (inject_residual) {
+    d->residual_layer = residual_layer;
+    d->residual_channels = residual_used;
+    d->residual_pitch = residual_pitch;
+    d->residual_pool = residual_pool ? 1 : 0;
+  }
+  d->save_residual = save_residual ? 1 : 0;
+  d->residual_out = output_residual_gpu.get();
   d->input = input_gpu, d->weights = filter_gpu.get(), d->thresholds = bn_gpu.get(), d->output = output_gpu.get();
 }
 
@@ -245,24 +354,24 @@ std::vector<uint32_t> Conv128LayerParam::download_output() const {
 
 // ---- Fc128LayerParam -------------------------------------------------------------------------------
 
-Fc128LayerParam::Fc128LayerParam(const char *name_, int batch_, int input_height_, int input_width_,
-                                 int input_channels_, int weight_width_, int a_bit_, int w_bit_)
-    : name(name_), batch(batch_), input_height(input_height_), input_width(input_width_),
-      input_channels(input_channels_), weight_width(weight_width_), a_bit(a_bit_), w_bit(w_bit_) {
-  in_cpad = pad_to(input_channels, 32);
+Fc128LayerParam::Fc128LayerParam(const char *name_, int input_height_, int input_width_, int weight_width_, int a_bit_,
+                                 int w_bit_)
+    : name(name_), input_height(input_height_), input_width(input_width_), weight_width(weight_width_), a_bit(a_bit_),
+      w_bit(w_bit_) {
+  if (input_width % 32 != 0) status = APNN_EUNSUPPORTED;  // rows are whole packed words
   out_cpad = pad_to(weight_width, 32);
 }
 
 int Fc128LayerParam::initialize(Rng &rng, const uint32_t *prev_layer_gpu, int path_) {
-  int rc = random_planes_gpu(rng, weight_gpu, weight_width * input_height * input_width, input_channels, in_cpad,
-                             w_bit);
+  if (status != 0) return status;
+  int rc = random_planes_gpu(rng, weight_gpu, weight_width, input_width, input_width, w_bit);
   if (rc != 0) return rc;
   const double amax = (double)((1 << a_bit) - 1), wmax = (double)((1 << w_bit) - 1);
   const double ex2 = amax * (2 * amax + 1) / 6.0, ew2 = (wmax * wmax + 2 * wmax) / 3.0;
-  const double sigma = std::sqrt((double)input_height * input_width * input_channels * ex2 * ew2);
+  const double sigma = std::sqrt((double)input_width * ex2 * ew2);
   const std::vector<int32_t> thr = random_thresholds(rng, weight_width, a_bit, 0.0, sigma);
   if (bn_gpu.upload(thr.data(), thr.size() * sizeof(int32_t)) != hipSuccess) return 1;
-  if (output_gpu.allocate((size_t)a_bit * batch * (out_cpad / 32) * 4) != hipSuccess) return 1;
+  if (output_gpu.allocate((size_t)a_bit * input_height * (out_cpad / 32) * 4) != hipSuccess) return 1;
   input_gpu = prev_layer_gpu;
   path = path_;
   return 0;
@@ -273,13 +382,13 @@ int FC_new_global(Fc128LayerParam *p, hipStream_t stream) {
   d.W = p->weight_gpu.get();
   d.X = p->input_gpu;
   d.O = p->output_gpu.get();
-  d.batch = p->batch;
-  d.H = p->input_height;
-  d.Wd = p->input_width;
-  d.cin_pad = p->in_cpad;
+  d.batch = p->input_height;
+  d.H = 1;
+  d.Wd = 1;
+  d.cin_pad = p->input_width;
   d.COUT = p->weight_width;
-  d.R = p->input_height;
-  d.S = p->input_width;
+  d.R = 1;
+  d.S = 1;
   d.stride = 1;
   d.pad = 0;
   d.halo = 0;
@@ -296,24 +405,20 @@ int FC_new_global(Fc128LayerParam *p, hipStream_t stream) {
 int Fc128LayerParam::forward(hipStream_t stream) { return FC_new_global(this, stream); }
 
 void Fc128LayerParam::describe(apnn_layer_desc *d) const {
-  std::memset(d, 0, sizeof(*d));
-  copy_name(d->name, name);
-  d->kind = APNN_LAYER_FC;
-  d->batch = batch;
-  d->in_h = input_height, d->in_w = input_width, d->in_c = input_channels, d->in_cpad = in_cpad;
+  clear_desc(d, name, APNN_LAYER_FC, input_height);
+  d->in_h = 1, d->in_w = 1, d->in_c = input_width, d->in_cpad = input_width;
   d->out_h = 1, d->out_w = 1, d->out_c = weight_width, d->out_cpad = out_cpad;
-  d->R = input_height, d->S = input_width, d->stride = 1, d->pad = 0;
+  d->R = 1, d->S = 1, d->stride = 1, d->pad = 0;
   d->a_bits = a_bit, d->w_bits = w_bit, d->out_bits = a_bit;
-  d->shortcut_layer = -1;
-  d->global_pool_shift = -1;
   d->input = input_gpu, d->weights = weight_gpu.get(), d->thresholds = bn_gpu.get(), d->output = output_gpu.get();
 }
 
 // ---- Out128LayerParam ------------------------------------------------------------------------------
 
-Out128LayerParam::Out128LayerParam(const char *name_, int batch_, int input_positions_, int input_channels_,
-                                   int weight_width_, int global_pool_shift_, int a_bit_)
-    : name(name_), batch(batch_), input_positions(input_positions_), input_channels(input_channels_),
+Out128LayerParam::Out128LayerParam(const char *name_, int input_height_, int input_width_, int weight_width_,
+                                   int a_bit_, int /*w_bit: the classifier's weights are int8*/, int input_positions_,
+                                   int global_pool_shift_)
+    : name(name_), batch(input_height_), input_positions(input_positions_), input_channels(input_width_),
       weight_width(weight_width_), global_pool_shift(global_pool_shift_), a_bit(a_bit_) {
   in_cpad = pad_to(input_channels, 32);
 }
@@ -349,15 +454,11 @@ int Output_new_global(Out128LayerParam *p, hipStream_t stream) {
 int Out128LayerParam::forward(hipStream_t stream) { return Output_new_global(this, stream); }
 
 void Out128LayerParam::describe(apnn_layer_desc *d) const {
-  std::memset(d, 0, sizeof(*d));
-  copy_name(d->name, name);
-  d->kind = APNN_LAYER_OUT_I8;
-  d->batch = batch;
+  clear_desc(d, name, APNN_LAYER_OUT_I8, batch);
   d->in_h = input_positions, d->in_w = 1, d->in_c = input_channels, d->in_cpad = in_cpad;
   d->out_h = 1, d->out_w = 1, d->out_c = weight_width, d->out_cpad = weight_width;
   d->R = 1, d->S = 1, d->stride = 1;
   d->a_bits = a_bit, d->w_bits = 8, d->out_bits = 32;
-  d->shortcut_layer = -1;
   d->global_pool_shift = global_pool_shift;
   d->input = input_gpu, d->weights = weight_gpu.get(), d->scale = scale_gpu.get(), d->bias = bias_gpu.get();
   d->output = output_gpu;
@@ -372,7 +473,8 @@ Network::~Network() {
 
 int Network::forward(const uint8_t *images, float *logits, hipStream_t stream) {
   if (images == nullptr || logits == nullptr) return APNN_ENULL;
-  first->set_input_gpu(images);
+  if (first != nullptr) first->set_input_gpu(images);
+  if (first_quant != nullptr) first_quant->set_input_gpu(images);
   last->set_output_gpu(logits);
   for (size_t i = 0; i < layers.size(); ++i) {
     // a residual block's first convolution and the downsample convolution listed right after it read

@@ -38,19 +38,20 @@ std::unique_ptr<Network> build_alexnet(int batch, uint64_t seed, int path) {
   net->first = c1;
   auto *c2 = add(*net, new Conv128LayerParam("Conv2", c1->output_height, c1->output_width, 5, 5, 64, 192, batch, 1, 1,
                                              true, 2, 2));
-  if (c2->initialize(rng, c1->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  if (c2->initialize(rng, c1->get_output_gpu(), nullptr, path)) return nullptr;
   auto *c3 = add(*net, new Conv128LayerParam("Conv3", c2->output_height, c2->output_width, 3, 3, 192, 384, batch));
-  if (c3->initialize(rng, c2->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  if (c3->initialize(rng, c2->get_output_gpu(), nullptr, path)) return nullptr;
   auto *c4 = add(*net, new Conv128LayerParam("Conv4", c3->output_height, c3->output_width, 3, 3, 384, 256, batch));
-  if (c4->initialize(rng, c3->get_output_gpu(), nullptr, 0, path)) return nullptr;
+  if (c4->initialize(rng, c3->get_output_gpu(), nullptr, path)) return nullptr;
   auto *c5 = add(*net, new Conv128LayerParam("Conv5", c4->output_height, c4->output_width, 3, 3, 256, 256, batch, 1, 1,
                                              true, 2, 2));
-  if (c5->initialize(rng, c4->get_output_gpu(), nullptr, 0, path)) return nullptr;
-  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, c5->output_height, c5->output_width, 256, 4096));
+  if (c5->initialize(rng, c4->get_output_gpu(), nullptr, path)) return nullptr;
+  // the FC layer consumes the batch-major feature map as it lies in memory: H*W*C features per image
+  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, c5->output_height * c5->output_width * c5->out_cpad, 4096));
   if (f1->initialize(rng, c5->get_output_gpu(), path)) return nullptr;
-  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 1, 1, 4096, 4096));
+  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 4096, 4096));
   if (f2->initialize(rng, f1->get_output_gpu(), path)) return nullptr;
-  auto *out = add(*net, new Out128LayerParam("Fout", batch, 1, 4096, 1000, -1));
+  auto *out = add(*net, new Out128LayerParam("Fout", batch, 4096, 1000));
   if (out->initialize(rng, f2->get_output_gpu(), nullptr)) return nullptr;
   net->last = out;
   return net;
@@ -75,17 +76,17 @@ std::unique_ptr<Network> build_vgg(int batch, uint64_t seed, int path) {
     snprintf(nm, sizeof nm, "Conv%d", i + 2);
     const int pool = (i == 2 || i == 5 || i == 8) ? 2 : 1;  // Conv4, Conv7, Conv10
     auto *c = add(*net, new Conv128LayerParam(nm, h, w, 3, 3, cin, chans[i], batch, 1, 1, true, pool, pool));
-    if (c->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+    if (c->initialize(rng, prev, nullptr, path)) return nullptr;
     prev = c->get_output_gpu();
     h = c->output_height;
     w = c->output_width;
     cin = chans[i];
   }
-  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, h, w, 512, 4096));
+  auto *f1 = add(*net, new Fc128LayerParam("Fc1", batch, h * w * 512, 4096));
   if (f1->initialize(rng, prev, path)) return nullptr;
-  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 1, 1, 4096, 4096));
+  auto *f2 = add(*net, new Fc128LayerParam("Fc2", batch, 4096, 4096));
   if (f2->initialize(rng, f1->get_output_gpu(), path)) return nullptr;
-  auto *out = add(*net, new Out128LayerParam("Fout", batch, 1, 4096, 1000, -1));
+  auto *out = add(*net, new Out128LayerParam("Fout", batch, 4096, 1000));
   if (out->initialize(rng, f2->get_output_gpu(), nullptr)) return nullptr;
   net->last = out;
   return net;
@@ -99,7 +100,7 @@ std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path) {
   auto net = std::make_unique<Network>();
   net->batch = batch;
   Rng rng(seed);
-  auto *stem = add(*net, new InConv128LayerParam("Conv1", 224, 224, 7, 7, 3, 64, batch, 2, 2, true, 3, 3, 2, 1));
+  auto *stem = add(*net, new InConv128LayerParam("Conv1", 224, 224, 7, 7, 3, 64, batch, 2, 2, true, 3, 3, false, 2, 1));
   if (stem->initialize(rng, nullptr)) return nullptr;
   net->first = stem;
   const uint32_t *prev = stem->get_output_gpu();
@@ -112,22 +113,22 @@ std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path) {
       char nm[16];
       snprintf(nm, sizeof nm, "L%dB%dC1", stage + 1, blk + 1);
       auto *c1 = add(*net, new Conv128LayerParam(nm, h, w, 3, 3, cin, ch, batch, stride, stride));
-      if (c1->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+      if (c1->initialize(rng, prev, nullptr, path)) return nullptr;
       const uint32_t *shortcut = prev;
       int shortcut_index = prev_index;
       if (stride != 1 || cin != ch) {
         snprintf(nm, sizeof nm, "L%dB%dDS", stage + 1, blk + 1);
         auto *ds = add(*net, new Conv128LayerParam(nm, h, w, 1, 1, cin, ch, batch, stride, stride, false));
-        if (ds->initialize(rng, prev, nullptr, 0, path)) return nullptr;
+        if (ds->initialize(rng, prev, nullptr, path)) return nullptr;
         ds->pairs_with_previous = true;  // same input as c1: launched together
         shortcut = ds->get_output_gpu();
         shortcut_index = (int)net->layers.size() - 1;
       }
       snprintf(nm, sizeof nm, "L%dB%dC2", stage + 1, blk + 1);
-      auto *c2 = add(*net, new Conv128LayerParam(nm, c1->output_height, c1->output_width, 3, 3, ch, ch, batch, 1, 1,
-                                                 true, 1, 1, false, false, true, ch));
-      if (c2->initialize(rng, c1->get_output_gpu(), shortcut, shortcut_scale_for(3, 3, ch, 2), path)) return nullptr;
-      c2->shortcut_layer = shortcut_index;
+      auto *c2 = add(*net, new Conv128LayerParam(nm, c1->output_height, c1->output_width, 3, 3, ch, ch, batch));
+      // the shortcut is the packed output of the block input (or of the downsample convolution)
+      c2->set_packed_shortcut(shortcut, shortcut_scale_for(3, 3, ch, 2), shortcut_index);
+      if (c2->initialize(rng, c1->get_output_gpu(), nullptr, path)) return nullptr;
       prev = c2->get_output_gpu();
       prev_index = (int)net->layers.size() - 1;
       h = c2->output_height;
@@ -135,8 +136,68 @@ std::unique_ptr<Network> build_resnet18(int batch, uint64_t seed, int path) {
       cin = ch;
     }
   }
-  auto *out = add(*net, new Out128LayerParam("Fc", batch, h * w, 512, 1000, 1));
+  auto *out = add(*net, new Out128LayerParam("Fc", batch, 512, 1000, 2, 1, h * w, 1));
   if (out->initialize(rng, prev, nullptr)) return nullptr;
+  net->last = out;
+  return net;
+}
+
+// The reference's ResNet18 demo with its own constructor argument lists
+// (APNN-TC-nn/src/resnet18.cu:40-142): the image is quantized to bit-planes (images_quantization), the stem
+// is a low-bit 7x7 stride-4 convolution that saves its int32 sums, every block's second convolution
+// injects the saved sums of the layer two convolutions back (and saves its own), max-pooled 2x2 and
+// limited to residual_channels where a stage halves the map; FC 7*7*512 -> 512 and 1000 outputs.
+// Differences forced by this build: thresholds are 2-bit (a_bit = 2, the reference's layers compare
+// against one float), and the output layer's weights are int8.
+std::unique_ptr<Network> build_resnet18_reference(int batch, uint64_t seed, int path) {
+  auto net = std::make_unique<Network>();
+  net->batch = batch;
+  Rng rng(seed);
+  auto *img = add(*net, new ImageQuantLayerParam("Image", batch, 224, 224, 3, 2));
+  if (img->initialize(nullptr)) return nullptr;
+  net->first_quant = img;
+  auto index_of_last = [&]() { return (int)net->layers.size() - 1; };
+
+  auto *bconv1 = add(*net, new Conv128LayerParam("Conv1", 224, 224, 7, 7, 3, 64, batch, 4, 4, true, 1, 1, true));
+  // resnet18.cu:40-41 passes `true` in the ahead_fc position with the comment "save residual", and
+  // l1b1c2 reads bconv1->get_output_residual_gpu(): the stem has to save its sums
+  bconv1->save_residual = true;
+  if (bconv1->initialize(rng, img->get_output_gpu(), nullptr, path)) return nullptr;
+
+  struct Saved {
+    const int32_t *gpu;
+    int channels, layer;
+  };
+  Saved saved{bconv1->get_output_residual_gpu(), 64, index_of_last()};
+  Conv128LayerParam *prev = bconv1;
+  // (input channels, output channels, stride of the first convolution, residual_channels / residual_pool of
+  // the second one), resnet18.cu:44-131
+  struct Block {
+    int cin, cout, stride, res_channels;
+    bool res_pool, ahead_fc, save;
+  };
+  const Block blocks[8] = {{64, 64, 1, 64, false, false, true},    {64, 64, 1, 128, false, false, true},
+                           {64, 128, 2, 128, true, false, true},   {128, 128, 1, 128, false, false, true},
+                           {128, 256, 2, 128, true, false, true},  {256, 256, 1, 256, false, false, true},
+                           {256, 512, 2, 256, true, false, true},  {512, 512, 1, 512, false, true, false}};
+  for (int i = 0; i < 8; ++i) {
+    const Block &b = blocks[i];
+    char nm[16];
+    snprintf(nm, sizeof nm, "L%dB%dC1", i / 2 + 1, i % 2 + 1);
+    auto *c1 = add(*net, new Conv128LayerParam(nm, prev->output_height, prev->output_width, 3, 3, b.cin, b.cout, batch,
+                                               b.stride, b.stride));
+    if (c1->initialize(rng, prev->get_output_gpu(), nullptr, path)) return nullptr;
+    snprintf(nm, sizeof nm, "L%dB%dC2", i / 2 + 1, i % 2 + 1);
+    auto *c2 = add(*net, new Conv128LayerParam(nm, c1->output_height, c1->output_width, 3, 3, b.cout, b.cout, batch, 1, 1,
+                                               true, 1, 1, b.ahead_fc, b.save, true, b.res_channels, b.res_pool));
+    if (c2->initialize(rng, c1->get_output_gpu(), saved.gpu, path, saved.channels, saved.layer)) return nullptr;
+    saved = Saved{c2->get_output_residual_gpu(), b.cout, index_of_last()};
+    prev = c2;
+  }
+  auto *fc = add(*net, new Fc128LayerParam("Fc1", batch, prev->output_height * prev->output_width * 512, 512));
+  if (fc->initialize(rng, prev->get_output_gpu(), path)) return nullptr;
+  auto *out = add(*net, new Out128LayerParam("Fout", batch, 512, 1000));
+  if (out->initialize(rng, fc->get_output_gpu(), nullptr)) return nullptr;
   net->last = out;
   return net;
 }
@@ -158,6 +219,8 @@ apnn_net *apnn_net_create(int kind, int batch, unsigned long long seed, int path
     n = apnn_nn::build_resnet18(batch, seed, path);
   } else if (kind == APNN_NET_VGG) {
     n = apnn_nn::build_vgg(batch, seed, path);
+  } else if (kind == APNN_NET_RESNET18_REFERENCE) {
+    n = apnn_nn::build_resnet18_reference(batch, seed, path);
   }
   if (!n) return nullptr;
   apnn_net *h = new (std::nothrow) apnn_net;

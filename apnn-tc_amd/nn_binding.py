@@ -5,11 +5,11 @@ import os
 from . import binding
 
 __all__ = ["NN_LIB_PATH", "nn_lib", "LayerDesc", "NET_ALEXNET", "NET_RESNET18", "NET_VGG",
-           "LAYER_INCONV_I8", "LAYER_CONV", "LAYER_FC", "LAYER_OUT_I8", "NN_DECLARED_SYMBOLS"]
+           "LAYER_INCONV_I8", "LAYER_CONV", "LAYER_FC", "LAYER_OUT_I8", "LAYER_IMAGE_QUANT", "NET_RESNET18_REFERENCE", "NN_DECLARED_SYMBOLS"]
 
 NN_LIB_PATH = os.path.join(binding.PKG_DIR, "lib", "libapnn_nn.so")
-NET_ALEXNET, NET_RESNET18, NET_VGG = 0, 1, 2
-LAYER_INCONV_I8, LAYER_CONV, LAYER_FC, LAYER_OUT_I8 = 0, 1, 2, 3
+NET_ALEXNET, NET_RESNET18, NET_VGG, NET_RESNET18_REFERENCE = 0, 1, 2, 3
+LAYER_INCONV_I8, LAYER_CONV, LAYER_FC, LAYER_OUT_I8, LAYER_IMAGE_QUANT = 0, 1, 2, 3, 4
 NN_DECLARED_SYMBOLS = ["apnn_net_create", "apnn_net_destroy", "apnn_net_forward", "apnn_net_forward_graph",
                        "apnn_net_layer_count", "apnn_net_layer", "apnn_net_bench", "apnn_nn_download"]
 
@@ -21,8 +21,9 @@ class LayerDesc(ctypes.Structure):
                 [(n, _ci) for n in ("kind", "batch", "in_h", "in_w", "in_c", "in_cpad", "out_h", "out_w", "out_c",
                                     "out_cpad", "R", "S", "stride", "pad", "pool_win", "pool_stride", "pool_pad",
                                     "a_bits", "w_bits", "out_bits", "shortcut_layer", "shortcut_scale",
-                                    "global_pool_shift")] +
-                [(n, _vp) for n in ("input", "weights", "thresholds", "scale", "bias", "output")])
+                                    "global_pool_shift", "residual_layer", "residual_channels", "residual_pitch",
+                                    "residual_pool", "save_residual")] +
+                [(n, _vp) for n in ("input", "weights", "thresholds", "scale", "bias", "output", "residual_out")])
 
 
 _lib = None

@@ -49,6 +49,88 @@ def gemm_bytes(M, N, K, wb, xb):
     return (wb * M * K + xb * N * K) // 8 + 4 * M * N
 
 
+def crossover_table(A, G, O, benchlib, stream):
+    """Every kernel path / tile shape pinned in turn on the shapes around which the library's own choice
+    (APNN_PATH_AUTO) changes: the M=64 sweep end point, the small-GEMM cross-over to the matrix cores,
+    large GEMMs, the 16x16 convolution family and the ResNet18 layer shapes at batch 8 and 64.  Each entry
+    lists the time of every candidate that is built, the library's choice (from apnn_*_plan) and how far
+    that choice is from the fastest candidate."""
+    import numpy as np
+    import torch
+    KN = {A.KERNEL_VALU_TILE: "valu", A.KERNEL_VALU_DIRECT: "valu-direct", A.KERNEL_MFMA_FP4: "fp4",
+          A.KERNEL_MFMA_I8: "i8", A.KERNEL_PATCH_FP4: "patch"}
+    rng = np.random.default_rng(0x5EED0004)
+
+    def run(desc, fn_graph, fn_plain, small):
+        ev, wall = ctypes.c_float(), ctypes.c_double()
+        if small:
+            rc = fn_graph(ctypes.byref(desc), 200, 1000, GRAPH_BATCH, ctypes.byref(ev), ctypes.byref(wall))
+            n = 1000
+        else:
+            rc = fn_plain(ctypes.byref(desc), 3, 20, stream, ctypes.byref(ev), ctypes.byref(wall))
+            n = 20
+        torch.cuda.synchronize()
+        return None if rc != 0 else ev.value / n * 1e3
+
+    def sweep(name, desc, plan_fn, fn_graph, fn_plain, small, cands):
+        plan = A.Plan()
+        desc.path = A.PATH_AUTO
+        assert plan_fn(ctypes.byref(desc), ctypes.byref(plan)) == 0
+        auto = "%s/%d" % (KN[plan.kernel], plan.tile)
+        times = {}
+        for pth, tile in cands:
+            desc.path = pth | ((tile + 1) << 8)
+            p2 = A.Plan()
+            if plan_fn(ctypes.byref(desc), ctypes.byref(p2)) != 0:
+                continue        # not built for this precision / load width, or does not fit
+            t = run(desc, fn_graph, fn_plain, small)
+            if t is not None:
+                times["%s/%d" % (KN[p2.kernel], p2.tile)] = round(t, 2)
+        desc.path = A.PATH_AUTO
+        t_auto = run(desc, fn_graph, fn_plain, small)
+        best = min(times, key=times.get)
+        return {"shape": name, "auto": auto, "auto_us": round(t_auto, 2), "best": best, "best_us": times[best],
+                "auto_over_best": round(t_auto / times[best], 3), "candidates_us": times}
+
+    L = A.lib()
+    out = []
+    gemm_cands = ([(A.PATH_VALU, t) for t in range(5)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 6)] +
+                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 6)])
+    for (wb, xb, M, N, K) in [(1, 2, 64, 1024, 1024), (1, 4, 64, 1024, 1024), (1, 2, 128, 128, 2048), (1, 2, 256, 256, 1024),
+                              (1, 2, 256, 256, 4096), (1, 2, 512, 512, 1024), (1, 2, 1024, 1024, 1024),
+                              (1, 2, 2048, 2048, 2048), (1, 4, 2048, 2048, 2048), (1, 2, 4096, 4096, 4096)]:
+        W = G.to_dev(O.random_planes(rng, wb, M, K // 32))
+        X = G.to_dev(O.random_planes(rng, xb, N, K // 32))
+        D = G.dev_empty_i32(M * N)
+        d = A.GemmDesc(W=W.data_ptr(), X=X.data_ptr(), D=D.data_ptr(), M=M, N=N, K=K, wb=wb, xb=xb)
+        cands = [c for c in gemm_cands if not (c[0] == A.PATH_VALU and M * N > 1024 * 1024 and c[1] != 0)]
+        out.append(sweep("gemm w%da%d %dx%dx%d" % (wb, xb, M, N, K), d, L.apnn_gemm_plan, benchlib.apnn_bench_gemm_graph,
+                         benchlib.apnn_bench_gemm, M * N <= 512 * 512, cands))
+    conv_cands = ([(A.PATH_VALU, t) for t in range(4)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 7)] +
+                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 3, 4, 7)] + [(A.PATH_MFMA_PATCH, t) for t in range(5)])
+    geoms = [("conv16 b1 C=%d" % c, 1, 16, c, c, 3, 1, 1) for c in (128, 512, 1024)]
+    geoms += [("conv16 b16 C=%d" % c, 16, 16, c, c, 3, 1, 1) for c in (128, 256, 512, 1024)]
+    for b in (8, 64):
+        geoms += [("resnet b%d 56x56 64->64" % b, b, 56, 64, 64, 3, 1, 1), ("resnet b%d 56x56 64->128 /2" % b, b, 56, 64, 128, 3, 2, 1),
+                  ("resnet b%d 28x28 128->128" % b, b, 28, 128, 128, 3, 1, 1), ("resnet b%d 28x28 128->256 /2" % b, b, 28, 128, 256, 3, 2, 1),
+                  ("resnet b%d 14x14 256->256" % b, b, 14, 256, 256, 3, 1, 1), ("resnet b%d 14x14 256->512 /2" % b, b, 14, 256, 512, 3, 2, 1),
+                  ("resnet b%d 7x7 512->512" % b, b, 7, 512, 512, 3, 1, 1), ("resnet b%d 56x56 64->128 1x1 /2" % b, b, 56, 64, 128, 1, 2, 0)]
+    for (name, batch, H, cin, cout, R, stride, pad) in geoms:
+        X = G.to_dev(O.random_planes(rng, 2, batch * H * H, cin // 32))
+        Wt = G.to_dev(O.random_planes(rng, 1, cout * R * R, cin // 32))
+        Ho = (H + 2 * pad - R) // stride + 1
+        thr = G.to_dev(np.sort(rng.integers(-200, 200, size=(cout, 3)), axis=1).astype(np.int32))
+        outp = G.dev_empty_i32(2 * batch * Ho * Ho * cout // 32)
+        E = G.epilogue(mode=A.EPI_BN, out_bits=2, thr=thr)
+        d = A.ConvDesc(W=Wt.data_ptr(), X=X.data_ptr(), O=outp.data_ptr(), batch=batch, H=H, Wd=H, cin_pad=cin, COUT=cout,
+                       R=R, S=R, stride=stride, pad=pad, halo=0, wb=1, xb=2, weight_mode=A.WEIGHT_SYMMETRIC, epi=E)
+        rows = batch * Ho * Ho
+        cands = [c for c in conv_cands if not (c[0] == A.PATH_VALU and rows * cout > 1024 * 1024 and c[1] != 0)]
+        out.append(sweep(name + " w1a2 bn-packed", d, L.apnn_conv_plan, benchlib.apnn_bench_conv_graph,
+                         benchlib.apnn_bench_conv, rows * cout <= 512 * 512, cands))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,8 +141,9 @@ def main():
     ap.add_argument("--extra", default="all",
                     help="comma list of secondary workloads to run after the headline: all, none, gemm_sweep, "
                          "gemm_large, gemm8192 (w1a2 only), conv, nets, resnet18_b8, resnet18_b64, alexnet_b8, "
-                         "alexnet_b64, vgg_b8, vgg_b64")
-    ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma"])
+                         "alexnet_b64, vgg_b8, vgg_b64; crossover (not part of all): every kernel path / tile "
+                         "pinned in turn on the shapes where the library's choice changes")
+    ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma", "mfma_i8"])
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one 256 MiB device copy (known traffic) for counter calibration")
     args = ap.parse_args()
@@ -93,7 +176,7 @@ def main():
                                           ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    path = {"auto": A.PATH_AUTO, "valu": A.PATH_VALU, "mfma": A.PATH_MFMA}[args.path]
+    path = {"auto": A.PATH_AUTO, "valu": A.PATH_VALU, "mfma": A.PATH_MFMA, "mfma_i8": A.PATH_MFMA_I8}[args.path]
 
     def make_inputs(M, N, K, wb, xb):
         W = O.random_planes(np.random.default_rng(0x5EED0001), wb, M, K // 32)
@@ -285,7 +368,7 @@ def main():
                     for C in ((128, 256, 384, 512, 640, 768, 896, 1024) if batch == 1 else (128, 256, 512, 1024)) \
                             if (w_, a_) == (1, 2) else (512, 1024):
                         for fused in (False, True):
-                            t = time_conv(batch, C, w_, a_, fused, 10, 200 if batch == 1 else 50)
+                            t = time_conv(batch, C, w_, a_, fused, 200 if batch == 1 else 10, 1000 if batch == 1 else 50)
                             t["shape"] = "w%da%d 3x3 16x16 b%d Cin=Cout=%d %s" % (
                                 w_, a_, batch, C, "bn-quantize packed out" if fused else "int32 out")
                             convs.append(t)
@@ -332,6 +415,8 @@ def main():
                 NL.apnn_net_destroy(net)
         if nets:
             extra["networks"] = nets
+    if "crossover" in want:
+        extra["crossover"] = crossover_table(A, G, O, benchlib, stream)
     result["extra"] = extra
 
     # ---- CPU baseline: the scalar oracle on the same inputs, host cores ---------------------------

@@ -21,13 +21,20 @@ extern "C" {
 
 enum { APNN_NET_ALEXNET = 0,   /* topology of APNN-TC-nn/src/alexnet.cu:42-81, int8 first conv / classifier */
        APNN_NET_RESNET18 = 1,  /* standard ResNet18 (3x3 basic blocks, strided 1x1 downsample convs)        */
-       APNN_NET_VGG = 2 };     /* topology of APNN-TC-nn/src/vgg.cu:49-127 (ten 3x3 convs, 96..512 channels,
+       APNN_NET_VGG = 2,       /* topology of APNN-TC-nn/src/vgg.cu:49-127 (ten 3x3 convs, 96..512 channels,
                                   first one stride 2; 2x2 pools after convs 1, 4, 7, 10; two 4096 FCs)       */
+       APNN_NET_RESNET18_REFERENCE = 3 }; /* the reference's own ResNet18 demo, layer for layer with its
+                                  constructor arguments (APNN-TC-nn/src/resnet18.cu:40-142): quantized image,
+                                  7x7 stride-4 low-bit stem, basic blocks whose shortcut is the saved int32 sum
+                                  of an earlier layer (max-pooled 2x2 and added to the first residual_channels
+                                  channels where the shape changes; no 1x1 convolutions), FC 25088->512, 1000
+                                  outputs */
 
 enum { APNN_LAYER_INCONV_I8 = 0, /* int8 conv + thresholds (+ max-pool) + pack                               */
        APNN_LAYER_CONV = 1,      /* low-bit conv, fused threshold / pool / shortcut epilogue                  */
        APNN_LAYER_FC = 2,        /* low-bit fully connected (a conv whose filter covers its whole input)      */
-       APNN_LAYER_OUT_I8 = 3 };  /* (global pool +) int8 classifier, float logits                             */
+       APNN_LAYER_OUT_I8 = 3,    /* (global pool +) int8 classifier, float logits                             */
+       APNN_LAYER_IMAGE_QUANT = 4 }; /* uint8 image -> bit-planes (code = pixel >> (8 - out_bits))            */
 
 typedef struct apnn_layer_desc {
   char name[16];
@@ -41,11 +48,17 @@ typedef struct apnn_layer_desc {
   int shortcut_layer;                  /* index of the layer whose packed output is the shortcut, -1 none */
   int shortcut_scale;
   int global_pool_shift;               /* OUT_I8: pooled = min(127, sum_of_codes >> shift); -1: no pooling */
+  int residual_layer;                  /* index of the layer whose saved int32 sums are injected, -1 none   */
+  int residual_channels;               /* the injected map is added to channels below this                  */
+  int residual_pitch;                  /* int32 values per pixel of the injected map                        */
+  int residual_pool;                   /* 1: the injected map is twice the size and max-pooled 2x2          */
+  int save_residual;                   /* 1: residual_out receives the int32 value the thresholds see       */
   const void *input;                   /* device pointers, valid for the lifetime of the network */
   const void *weights;                 /* CONV/FC: packed planes [w][cout][R][S][in_cpad/32]; I8: [cout][R][S][in_c] */
   const void *thresholds;              /* [out_c][2^out_bits-1] int32 */
   const void *scale, *bias;            /* OUT_I8: float [out_c] */
   const void *output;                  /* packed planes [out_bits][batch*out_h*out_w][out_cpad/32]; OUT_I8: float */
+  const void *residual_out;            /* save_residual: int32 [batch*conv_h*conv_w][out_c] (before pooling)  */
 } apnn_layer_desc;
 
 typedef struct apnn_net apnn_net;

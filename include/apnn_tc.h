@@ -227,6 +227,24 @@ int apnn_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, apnn_stream
 int apnn_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
                        float max_v, apnn_stream_t s);
 
+/* uint8 samples (raw image bytes) -> bit-planes: code = value >> (8 - bits), a uniform 2^bits-level
+ * quantizer of [0, 256), then the Bit_compression layout.  What images_quantization
+ * (APNN-TC-nn/src/kernel.cuh:129-161) does for a float image, for the uint8 images the networks here take. */
+int apnn_quantize_pack_u8(const uint8_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
+                          apnn_stream_t s);
+
+/* Float rows -> one bit-plane, bit = value >= 0, MSB-first: the input layer of the reference's fully
+ * connected networks (In128Layer, APNN-TC-nn/src/kernel.cuh:321-340).  planes:[rows][cpad/32]. */
+int apnn_binarize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, apnn_stream_t s);
+
+/* int32 shortcut map saved by an earlier layer (apnn_epilogue.save_acc) -> the `residual` operand of a
+ * later layer: the residual is added to channels below `channels` only and, with pool = 1, is the 2x2
+ * maximum of a source map of twice the height and width (inject_residual / residual_channels /
+ * residual_pool of Conv128Layer, APNN-TC-nn/src/kernel.cuh:779-831).
+ * in:[B][Ho*(1+pool)][Wo*(1+pool)][in_pitch] -> out:[B][Ho][Wo][out_channels], zero at channels >= `channels`. */
+int apnn_residual_prepare(const int32_t *in, int32_t *out, int B, int Ho, int Wo, int in_pitch, int channels,
+                          int out_channels, int pool, apnn_stream_t s);
+
 /* Host-side preparation (no device work): fold a batch-norm + uniform activation quantizer into the
  * integer thresholds of APNN_EPI_BN.  With y(v) = gamma[c] * (v * in_scale - mean[c]) / sqrt(var[c] + eps)
  * + beta[c] evaluated in double precision, code = clamp(floor(y / step), 0, 2^bits - 1) equals

@@ -60,7 +60,13 @@ def _check_network(G, kind, batch, path, graph):
         for i, d in enumerate(descs):
             nt = (1 << d.out_bits) - 1 if d.kind != A.LAYER_OUT_I8 else 0
             name = d.name.decode()
-            if d.kind == A.LAYER_INCONV_I8:
+            if d.kind == A.LAYER_IMAGE_QUANT:
+                rows = batch * d.in_h * d.in_w
+                codes = (images.reshape(rows, d.in_c) >> (8 - d.out_bits)).astype(np.uint32)
+                expect = O.pack_bits(codes, rows, d.in_c, d.out_cpad, d.out_bits)
+                got = _download(L, d.output, expect.size, np.uint32).reshape(expect.shape)
+                assert np.array_equal(got, expect), name
+            elif d.kind == A.LAYER_INCONV_I8:
                 Wt = _download(L, d.weights, d.out_c * d.R * d.S * d.in_c, np.int8).reshape(d.out_c, d.R, d.S, d.in_c)
                 thr = _download(L, d.thresholds, d.out_c * nt, np.int32).reshape(d.out_c, nt)
                 x = (images.astype(np.int16) - 128).astype(np.int8)
@@ -86,6 +92,23 @@ def _check_network(G, kind, batch, path, graph):
                     sp = _download(L, sd.output, sd.out_bits * srows * (sd.out_cpad // 32), np.uint32)
                     sc = O.unpack_bits(sp, srows, sd.out_c, sd.out_cpad, sd.out_bits).astype(np.int32)
                     acc = acc + d.shortcut_scale * sc.reshape(acc.shape)
+                if d.residual_layer >= 0:
+                    # int32 sums saved by an earlier layer: max-pooled 2x2 where this layer's map is half the
+                    # size, added to the first residual_channels channels (APNN-TC-nn/src/kernel.cuh:779-831)
+                    sd = descs[d.residual_layer]
+                    assert sd.save_residual and sd.out_c == d.residual_pitch, name
+                    f = 2 if d.residual_pool else 1
+                    Hc, Wc = acc.shape[1], acc.shape[2]
+                    assert (sd.out_h, sd.out_w) == (f * Hc, f * Wc), name
+                    src = _download(L, sd.residual_out, batch * sd.out_h * sd.out_w * sd.out_c, np.int32)
+                    src = src.reshape(batch, sd.out_h, sd.out_w, sd.out_c)
+                    if d.residual_pool:
+                        src = src.reshape(batch, Hc, 2, Wc, 2, sd.out_c).max(axis=(2, 4))
+                    acc = acc.copy()
+                    acc[..., :d.residual_channels] += src[..., :d.residual_channels]
+                if d.save_residual:
+                    saved = _download(L, d.residual_out, acc.size, np.int32).reshape(acc.shape)
+                    assert np.array_equal(saved, acc), name + " (saved residual)"
                 codes = O.bn_quantize(acc.reshape(-1, d.out_c), None, thr, None, d.out_bits).reshape(acc.shape)
                 if d.pool_win:
                     codes = O.maxpool2x2(codes)
@@ -128,6 +151,16 @@ def test_alexnet_and_vgg_batch8(G, kind, layers):
     net = G.A.NET_ALEXNET if kind == "alexnet" else G.A.NET_VGG
     assert _check_network(G, net, 8, 0, graph=False) == layers
     assert _check_network(G, net, 8, 0, graph=True) == layers
+
+
+@pytest.mark.parametrize("batch,path,graph", [(2, 0, False), (2, 1, False), (2, 2, False), (8, 0, True)])
+def test_reference_style_resnet18(G, batch, path, graph):
+    """The reference's own ResNet18 demo, built from its constructor argument lists
+    (APNN-TC-nn/src/resnet18.cu:40-142): save_residual / inject_residual / residual_channels /
+    residual_pool / ahead_fc all take part, and every layer -- the saved int32 maps included -- is
+    compared with the oracle."""
+    n = _check_network(G, G.A.NET_RESNET18_REFERENCE, batch, path, graph=graph)
+    assert n == 1 + 1 + 16 + 1 + 1      # image quantizer, stem, 16 block convolutions, FC, output
 
 
 @pytest.mark.parametrize("path", [0, 1, 2])

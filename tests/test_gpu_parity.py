@@ -736,6 +736,43 @@ def test_any_precision_descriptor_paths(G, wb, xb, ob, sym):
         G.run_conv(Wc, Xc, cin_pad=C, sym=sym, path=4, **kw)
 
 
+@pytest.mark.parametrize("rows,C,cpad", [(37, 3, 32), (50, 70, 128), (8, 256, 256)])
+def test_quantize_pack_u8_and_binarize(G, rows, C, cpad):
+    """uint8 samples -> top bits as codes -> planes; float rows -> one plane of (x >= 0) (In128Layer)."""
+    rng = np.random.default_rng(6100 + rows)
+    v = rng.integers(0, 256, size=(rows, C), dtype=np.uint8)
+    dV = torch.from_numpy(v).cuda()
+    for bits in (1, 2, 3, 8):
+        planes = G.dev_empty_i32(bits * rows * cpad // 32, fill=-7)
+        G.A.check(G.A.lib().apnn_quantize_pack_u8(G.ptr(dV), G.ptr(planes), rows, C, cpad, bits, None), "quantize_pack_u8")
+        expect = O.pack_bits((v >> (8 - bits)).astype(np.uint32), rows, C, cpad, bits)
+        assert np.array_equal(G.to_host(planes, np.uint32).reshape(expect.shape), expect)
+    x = rng.normal(size=(rows, C)).astype(np.float32)
+    x[0, :3] = [0.0, -0.0, np.float32(-1e-30)]
+    dX = torch.from_numpy(x).cuda()
+    planes = G.dev_empty_i32(rows * cpad // 32, fill=-7)
+    G.A.check(G.A.lib().apnn_binarize_pack(G.ptr(dX), G.ptr(planes), rows, C, cpad, None), "binarize_pack")
+    expect = O.pack_bits((x >= 0).astype(np.uint32), rows, C, cpad, 1)
+    assert np.array_equal(G.to_host(planes, np.uint32).reshape(expect.shape), expect)
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("B,Ho,Wo,pitch,channels,cout", [(2, 7, 5, 64, 64, 64), (3, 4, 6, 128, 64, 128), (1, 3, 3, 40, 33, 70),
+                                                     (2, 14, 14, 128, 128, 256)])
+def test_residual_prepare(G, B, Ho, Wo, pitch, channels, cout, pool):
+    rng = np.random.default_rng(6200 + Ho + cout + pool)
+    f = 2 if pool else 1
+    src = rng.integers(-50000, 50000, size=(B, Ho * f, Wo * f, pitch)).astype(np.int32)
+    d_in = G.to_dev(src)
+    d_out = G.dev_empty_i32(B * Ho * Wo * cout, fill=-7)
+    G.A.check(G.A.lib().apnn_residual_prepare(G.ptr(d_in), G.ptr(d_out), B, Ho, Wo, pitch, channels, cout, pool, None),
+              "residual_prepare")
+    m = src.reshape(B, Ho, 2, Wo, 2, pitch).max(axis=(2, 4)) if pool else src
+    expect = np.zeros((B, Ho, Wo, cout), np.int32)
+    expect[..., :channels] = m[..., :channels]
+    assert np.array_equal(G.to_host(d_out).reshape(expect.shape), expect)
+
+
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("rows,C,cpad", [(37, 3, 32), (50, 70, 128), (8, 256, 256)])
 def test_quantize_pack(G, bits, rows, C, cpad):
