@@ -7,7 +7,7 @@ __all__ = [
     "LIB_PATH", "lib", "build", "Epilogue", "GemmDesc", "ConvDesc", "Plan", "ApnnError", "check",
     "KERNEL_VALU_TILE", "KERNEL_VALU_DIRECT", "KERNEL_MFMA_FP4", "KERNEL_MFMA_I8", "KERNEL_PATCH_FP4",
     "EPI_INT32", "EPI_LOWBITS", "EPI_BN", "POOL_NONE", "POOL_AVG2X2", "POOL_MAX2X2",
-    "PATH_AUTO", "PATH_VALU", "PATH_MFMA", "PATH_MFMA_I8", "PATH_MFMA_PATCH", "WEIGHT_UNSIGNED", "WEIGHT_SYMMETRIC",
+    "PATH_AUTO", "PATH_VALU", "PATH_MFMA", "PATH_MFMA_I8", "PATH_MFMA_PATCH", "PATH_MFMA_XS", "KERNEL_MFMA_FP4_XS", "WEIGHT_UNSIGNED", "WEIGHT_SYMMETRIC",
     "OK", "EINVAL", "ENULL", "EALIGN", "EUNSUPPORTED", "DECLARED_SYMBOLS",
 ]
 
@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(PKG_DIR, "lib", "libapnn_tc.so")
 
 EPI_INT32, EPI_LOWBITS, EPI_BN = 0, 1, 2
 POOL_NONE, POOL_AVG2X2, POOL_MAX2X2 = 0, 1, 2
-PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_MFMA_I8, PATH_MFMA_PATCH = 0, 1, 2, 3, 4
+PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_MFMA_I8, PATH_MFMA_PATCH, PATH_MFMA_XS = 0, 1, 2, 3, 4, 5
 WEIGHT_UNSIGNED, WEIGHT_SYMMETRIC = 0, 1
 OK, EINVAL, ENULL, EALIGN, EUNSUPPORTED = 0, -1, -2, -3, -4
 
@@ -47,7 +47,7 @@ class Plan(ctypes.Structure):
                 ("split_k", _ci), ("workgroups", ctypes.c_longlong), ("patch_pixels", _ci), ("fp4_exact", _ci)]
 
 
-KERNEL_VALU_TILE, KERNEL_VALU_DIRECT, KERNEL_MFMA_FP4, KERNEL_MFMA_I8, KERNEL_PATCH_FP4 = 0, 1, 2, 3, 4
+KERNEL_VALU_TILE, KERNEL_VALU_DIRECT, KERNEL_MFMA_FP4, KERNEL_MFMA_I8, KERNEL_PATCH_FP4, KERNEL_MFMA_FP4_XS = 0, 1, 2, 3, 4, 5
 
 _GEMM_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci, _vp]
 _CONV_SIG = [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]

@@ -126,6 +126,41 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   return nullptr;
 }
 
+valu_fn mfmaxs_gemm_fn(int wb, int xb) {
+  if (wb == 1 && xb == 2) return apnn::mfmaxs_gemm_1_2_x;
+  if (wb == 1 && xb == 3) return apnn::mfmaxs_gemm_1_3_x;
+  if (wb == 1 && xb == 4) return apnn::mfmaxs_gemm_1_4_x;
+  if (wb == 2 && xb == 2) return apnn::mfmaxs_gemm_2_2_x;
+  return nullptr;
+}
+
+valu_fn mfmaxs_conv_fn(int xb, int wb) {
+  if (xb == 2 && wb == 1) return apnn::mfmaxs_conv_2_1_x;
+  if (xb == 3 && wb == 1) return apnn::mfmaxs_conv_3_1_x;
+  if (xb == 4 && wb == 1) return apnn::mfmaxs_conv_4_1_x;
+  if (xb == 2 && wb == 2) return apnn::mfmaxs_conv_2_2_x;
+  return nullptr;
+}
+
+// Tile of the expand-while-staging kernel: the largest of its shapes that still gives every compute
+// unit a work-group (1.5 per unit for 128x128, as for the other matrix-core kernel), else 64x64.
+int choose_xs_tile(int rowsA, int rowsB, bool conv) {
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;
+  auto ntiles = [&](int t) {
+    return (long long)((rowsA + apnn::kMfmaTileA[t] - 1) / apnn::kMfmaTileA[t]) *
+           ((rowsB + apnn::kMfmaTileB[t] - 1) / apnn::kMfmaTileB[t]);
+  };
+  auto fill = [&](int t) {
+    return (double)rowsA * rowsB / ((double)ntiles(t) * apnn::kMfmaTileA[t] * apnn::kMfmaTileB[t]);
+  };
+  const int big = conv ? 7 : 6;
+  if (rowsB > 64 && ntiles(big) >= cus && fill(big) >= 0.8) return big;
+  if (rowsB > 64 && 2 * ntiles(1) >= 3 * cus && fill(1) >= 0.8) return 1;
+  if (ntiles(3) >= cus && fill(3) >= 0.8) return 3;
+  return 2;
+}
+
 // The FP4 matrix-core kernels accumulate in fp32: every partial sum is a multiple of 1/4 and stays
 // exact while the largest possible result, K * (2^w - 1) * (2^a - 1), is below 2^24.
 bool fp4_exact(long long kwords, int wb, int xb) {
@@ -273,10 +308,17 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, b
   if (rowsB > 64) {
     const int big = conv ? 7 : 6;
     if (ntiles(big) >= cus && fill(big) >= 0.8) return big;
+    // 128x128 wants more than one work-group per compute unit (measured: with exactly one, the 128x64
+    // tile's two work-groups per compute unit are 4-9 % faster, GEMM 2048^3 and convolution 4096 x 1024)
+    if (2 * ntiles(1) >= 3 * cus && fill(1) >= 0.8) return 1;
+    if (ntiles(3) >= cus && fill(3) >= 0.8) return 3;
     if (ntiles(1) >= cus && fill(1) >= 0.8) return 1;
-    // convolution: 128 pixels x 64 channels per work-group (one activation expansion feeds two
-    // blocks per wave) measures faster than 64x64 whenever it still fills the chip
-    if (conv && ntiles(3) >= cus && fill(3) >= 0.8) return 3;
+  }
+  if (!conv) {
+    // GEMM entry points with few 64x64 tiles (measured at 512^2 and 1024^2 outputs over 1024 bits): the
+    // split-K tiles, one 32x32 block per work-group while that fills the chip once, 32x64 up to twice
+    if (KW >= 32 && ntiles(4) <= cus) return 4;
+    if (KW >= 32 && ntiles(5) <= 2 * cus) return 5;
   }
   if (ntiles(2) >= cus / 2 || KW < 16) return 2;
   return ntiles(5) >= cus / 2 ? 5 : 4;
@@ -352,7 +394,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff, tile_pin = (d->path >> 8) & 0xff;
-  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_PATCH))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_XS))
     return APNN_EINVAL;
   if ((rc = check_epilogue(d->epi, d->N, false, 0, 0))) return rc;
 
@@ -373,13 +415,34 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   p.planesB = d->xb;
   const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
-  if (path == APNN_PATH_MFMA && !f4ok) return APNN_EUNSUPPORTED;  // fp32 accumulation would round
+  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_XS) && !f4ok) return APNN_EUNSUPPORTED;  // fp32 would round
+  if (path == APNN_PATH_MFMA_XS) {
+    valu_fn fn = mfmaxs_gemm_fn(d->wb, d->xb);
+    if (fn == nullptr) return APNN_EUNSUPPORTED;
+    tile = tile_pin == 0 ? choose_xs_tile(p.rowsA, p.rowsB, false) : tile_pin - 1;
+    if (tile >= apnn::kMfmaTileCount) return APNN_EINVAL;
+    if (!apnn::mfma_xs_tile_enabled(false, 4, tile)) return APNN_EUNSUPPORTED;
+    if (plan != nullptr)
+      return fill_plan(plan, APNN_PATH_MFMA_XS, APNN_KERNEL_MFMA_FP4_XS, tile, apnn::kMfmaTileA[tile],
+                       apnn::kMfmaTileB[tile], 1, p, 0, f4ok);
+    return from_hip(fn(4, tile, p, stream));
+  }
   if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
     // AUTO: FP4 operands while their fp32 accumulation is exact, the int8 core (int32 accumulate) beyond
     const bool i8 = path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && !f4ok);
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, i8);
     if (fn != nullptr) {
       if ((rc = pick_mfma_tile(tile_pin, p, false, 4, i8, &tile))) return rc;
+      // Four activation planes on the largest tile: the kernel that expands operands while staging reuses
+      // every 16-byte LDS operand for two digit pairs and measures 8 % faster at 8192^3 (w1a4); with fewer
+      // planes it is bound by LDS bandwidth and loses (see mfma_xs_kernel.h)
+      if (path == APNN_PATH_AUTO && !i8 && tile == apnn::MT_256x128 && d->wb == 1 && d->xb == 4) {
+        valu_fn xs = mfmaxs_gemm_fn(d->wb, d->xb);
+        if (plan != nullptr)
+          return fill_plan(plan, APNN_PATH_MFMA_XS, APNN_KERNEL_MFMA_FP4_XS, tile, apnn::kMfmaTileA[tile],
+                           apnn::kMfmaTileB[tile], 1, p, 0, f4ok);
+        return from_hip(xs(4, tile, p, stream));
+      }
       if (plan != nullptr) {
         // a pinned tile that is not built is reported by the launcher; mirror that here
         return apnn::mfma_tile_enabled(i8 ? apnn::CORE_I8 : apnn::CORE_F4, false, 4, tile, d->wb, d->xb)
@@ -417,7 +480,7 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   if (d->wb < 1 || d->xb < 1 || d->wb > 8 || d->xb > 8) return APNN_EINVAL;
   if (d->weight_mode != APNN_WEIGHT_UNSIGNED && d->weight_mode != APNN_WEIGHT_SYMMETRIC) return APNN_EINVAL;
   const int path = d->path & 0xff;
-  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_PATCH))
+  if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_XS))
     return APNN_EINVAL;
   if (d->H + 2 * d->pad < d->R || d->Wd + 2 * d->pad < d->S) return APNN_EINVAL;
   const int Ho = (d->H + 2 * d->pad - d->R) / d->stride + 1;
@@ -490,7 +553,19 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream, apnn_plan *plan = null
       return plan != nullptr ? plan_direct(plan, p, f4ok) : from_hip(vf(vw, apnn::TILE_DIRECT, p, stream));
   }
   // fp32 accumulation of the FP4 kernels would round: pinned FP4 paths refuse, AUTO moves on
-  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_PATCH) && !f4ok) return APNN_EUNSUPPORTED;
+  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_PATCH || path == APNN_PATH_MFMA_XS) && !f4ok)
+    return APNN_EUNSUPPORTED;
+  if (path == APNN_PATH_MFMA_XS) {
+    valu_fn fn = mfmaxs_conv_fn(d->xb, d->wb);
+    if (fn == nullptr) return APNN_EUNSUPPORTED;
+    tile = tile_pin == 0 ? choose_xs_tile(p.rowsA, p.rowsB, true) : tile_pin - 1;
+    if (tile >= apnn::kMfmaTileCount) return APNN_EINVAL;
+    if (!apnn::mfma_xs_tile_enabled(true, vw, tile)) return APNN_EUNSUPPORTED;
+    if (plan != nullptr)
+      return fill_plan(plan, APNN_PATH_MFMA_XS, APNN_KERNEL_MFMA_FP4_XS, tile, apnn::kMfmaTileA[tile],
+                       apnn::kMfmaTileB[tile], 1, p, 0, f4ok);
+    return from_hip(fn(vw, tile, p, stream));
+  }
   if (path == APNN_PATH_MFMA_PATCH || (path == APNN_PATH_AUTO && f4ok)) {
     patch_fn pf = patch_conv_fn(d->xb, d->wb);
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);

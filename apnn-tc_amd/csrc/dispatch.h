@@ -47,6 +47,17 @@ APNN_DECL_MFMA4(conv, 3, 1)
 APNN_DECL_MFMA4(conv, 4, 1)
 APNN_DECL_MFMA4(conv, 2, 2)
 #undef APNN_DECL_MFMA
+#define APNN_DECL_MFMAXS(kind, pa, pb) \
+  hipError_t mfmaxs_##kind##_##pa##_##pb##_x(int vw, int tile, const KParams &p, hipStream_t s);
+APNN_DECL_MFMAXS(gemm, 1, 2)
+APNN_DECL_MFMAXS(gemm, 1, 3)
+APNN_DECL_MFMAXS(gemm, 1, 4)
+APNN_DECL_MFMAXS(gemm, 2, 2)
+APNN_DECL_MFMAXS(conv, 2, 1)
+APNN_DECL_MFMAXS(conv, 3, 1)
+APNN_DECL_MFMAXS(conv, 4, 1)
+APNN_DECL_MFMAXS(conv, 2, 2)
+#undef APNN_DECL_MFMAXS
 #define APNN_DECL_PATCH(pa, pb) hipError_t patch_conv_##pa##_##pb##_x(int tile, const KParams &p, hipStream_t s);
 APNN_DECL_PATCH(2, 1)
 APNN_DECL_PATCH(3, 1)
@@ -88,6 +99,13 @@ constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile, int pa, 
   if (!conv) return tile != MT_256x256 && tile != MT_128x256;
   if (vw == 1) return tile == MT_64x64 || tile == MT_32x32_K4;
   return tile != MT_256x256 && tile != MT_256x128;
+}
+
+// tiles of the kernel that expands operands while staging (mfma_xs_kernel.h), by their MfmaTile index:
+// the shapes whose four waves tile the output; convolution with 128-bit loads only
+constexpr bool mfma_xs_tile_enabled(bool conv, int vw, int tile) {
+  if (conv) return vw == 4 && (tile == MT_128x128 || tile == MT_64x64 || tile == MT_128x64 || tile == MT_128x256);
+  return tile == MT_128x128 || tile == MT_64x64 || tile == MT_128x64 || tile == MT_256x128;
 }
 
 // tile shapes of the patch-resident convolution kernel, index = enum PatchTile in patch_conv_kernel.h

@@ -58,7 +58,7 @@ def crossover_table(A, G, O, benchlib, stream):
     import numpy as np
     import torch
     KN = {A.KERNEL_VALU_TILE: "valu", A.KERNEL_VALU_DIRECT: "valu-direct", A.KERNEL_MFMA_FP4: "fp4",
-          A.KERNEL_MFMA_I8: "i8", A.KERNEL_PATCH_FP4: "patch"}
+          A.KERNEL_MFMA_I8: "i8", A.KERNEL_PATCH_FP4: "patch", A.KERNEL_MFMA_FP4_XS: "xs"}
     rng = np.random.default_rng(0x5EED0004)
 
     def run(desc, fn_graph, fn_plain, small):
@@ -95,10 +95,11 @@ def crossover_table(A, G, O, benchlib, stream):
     L = A.lib()
     out = []
     gemm_cands = ([(A.PATH_VALU, t) for t in range(5)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 6)] +
-                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 6)])
+                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 6)] + [(A.PATH_MFMA_XS, t) for t in (1, 2, 3, 6)])
     for (wb, xb, M, N, K) in [(1, 2, 64, 1024, 1024), (1, 4, 64, 1024, 1024), (1, 2, 128, 128, 2048), (1, 2, 256, 256, 1024),
                               (1, 2, 256, 256, 4096), (1, 2, 512, 512, 1024), (1, 2, 1024, 1024, 1024),
-                              (1, 2, 2048, 2048, 2048), (1, 4, 2048, 2048, 2048), (1, 2, 4096, 4096, 4096)]:
+                              (1, 2, 2048, 2048, 2048), (1, 4, 2048, 2048, 2048), (1, 2, 4096, 4096, 4096),
+                              (1, 4, 4096, 4096, 4096), (1, 2, 8192, 8192, 8192), (2, 2, 8192, 8192, 8192)]:
         W = G.to_dev(O.random_planes(rng, wb, M, K // 32))
         X = G.to_dev(O.random_planes(rng, xb, N, K // 32))
         D = G.dev_empty_i32(M * N)
@@ -107,7 +108,8 @@ def crossover_table(A, G, O, benchlib, stream):
         out.append(sweep("gemm w%da%d %dx%dx%d" % (wb, xb, M, N, K), d, L.apnn_gemm_plan, benchlib.apnn_bench_gemm_graph,
                          benchlib.apnn_bench_gemm, M * N <= 512 * 512, cands))
     conv_cands = ([(A.PATH_VALU, t) for t in range(4)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 7)] +
-                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 3, 4, 7)] + [(A.PATH_MFMA_PATCH, t) for t in range(5)])
+                  [(A.PATH_MFMA_I8, t) for t in (1, 2, 3, 4, 7)] + [(A.PATH_MFMA_PATCH, t) for t in range(5)] +
+                  [(A.PATH_MFMA_XS, t) for t in (1, 2, 3, 7)])
     geoms = [("conv16 b1 C=%d" % c, 1, 16, c, c, 3, 1, 1) for c in (128, 512, 1024)]
     geoms += [("conv16 b16 C=%d" % c, 16, 16, c, c, 3, 1, 1) for c in (128, 256, 512, 1024)]
     for b in (8, 64):
@@ -144,6 +146,9 @@ def main():
                          "alexnet_b64, vgg_b8, vgg_b64; crossover (not part of all): every kernel path / tile "
                          "pinned in turn on the shapes where the library's choice changes")
     ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma", "mfma_i8"])
+    ap.add_argument("--shape", action="append", default=[],
+                    help="extra workload on --path (repeatable; used by the profile commands): "
+                         "gemm:w1a2:M:N:K or conv:w1a2:b16:c1024:int32|fused (3x3 on a 16x16 map)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one 256 MiB device copy (known traffic) for counter calibration")
     args = ap.parse_args()
@@ -415,6 +420,23 @@ def main():
                 NL.apnn_net_destroy(net)
         if nets:
             extra["networks"] = nets
+    for spec in args.shape:
+        f = spec.split(":")
+        w_, a_ = int(f[1][1]), int(f[1][3])
+        if f[0] == "gemm":
+            Mg, Ng, Kg = int(f[2]), int(f[3]), int(f[4])
+            small = Mg * Ng <= 512 * 512
+            vr = None if Mg * Ng <= 1024 * 1024 else [0, Mg // 2 + 1, Mg - 1]
+            t = time_gemm(Mg, Ng, Kg, w_, a_, A.WEIGHT_UNSIGNED, 200 if small else 2, 2000 if small else 5,
+                          verify_rows=vr, graph=small)
+            tt = 2.0 * Mg * Ng * Kg / (t["event_ms"] * 1e-3) / 1e12
+            extra.setdefault("requested", []).append({"shape": spec, "path": args.path, "us": round(t["event_ms"] * 1e3, 3),
+                                                      "tops": round(tt, 2), "verified": t["verified"]})
+        else:
+            bt, Cc = int(f[2][1:]), int(f[3][1:])
+            t = time_conv(bt, Cc, w_, a_, f[4] == "fused", 200 if bt == 1 else 10, 1000 if bt == 1 else 50)
+            t.update(shape=spec, path=args.path)
+            extra.setdefault("requested", []).append(t)
     if "crossover" in want:
         extra["crossover"] = crossover_table(A, G, O, benchlib, stream)
     result["extra"] = extra

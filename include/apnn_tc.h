@@ -115,9 +115,12 @@ enum { APNN_PATH_AUTO = 0,
                                   accumulation, exact while K*(2^wb-1)*(2^xb-1) < 2^24: beyond that a
                                   pinned FP4 path returns APNN_EUNSUPPORTED and AUTO uses the int8 core   */
        APNN_PATH_MFMA_I8 = 3,  /* planes expanded to int8 operands of v_mfma_i32_32x32x32_i8         */
-       APNN_PATH_MFMA_PATCH = 4 };/* convolution only: FP4 matrix-core path with the tile's input patch
+       APNN_PATH_MFMA_PATCH = 4,/* convolution only: FP4 matrix-core path with the tile's input patch
                                   expanded once into LDS and read in place by every filter tap;
                                   APNN_EUNSUPPORTED when the patch or filter block does not fit   */
+       APNN_PATH_MFMA_XS = 5 };/* FP4 matrix-core path whose staging threads expand the planes, so that
+                                  LDS holds ready operands (tiles 128x128, 64x64, 128x64 and 256x128 /
+                                  128x256; w1a2, w1a3, w1a4, w2a2; convolution needs cin_pad % 128 == 0) */
 /* `path` fields: low byte = APNN_PATH_*; bits 8..15 = 0 (library picks the tile shape) or
  * 1 + tile index to pin it (tuning / test coverage of every tile shape; APNN_EINVAL if the
  * chosen kernel family has no such tile or the epilogue cannot use it). */
@@ -187,7 +190,8 @@ enum { APNN_KERNEL_VALU_TILE = 0,   /* LDS-tiled popcount kernel                
        APNN_KERNEL_VALU_DIRECT = 1, /* register-only popcount kernel (small GEMMs, FC layers)         */
        APNN_KERNEL_MFMA_FP4 = 2,
        APNN_KERNEL_MFMA_I8 = 3,
-       APNN_KERNEL_PATCH_FP4 = 4 };
+       APNN_KERNEL_PATCH_FP4 = 4,
+       APNN_KERNEL_MFMA_FP4_XS = 5 };
 typedef struct apnn_plan {
   int path;              /* APNN_PATH_* taken (never AUTO) */
   int kernel;            /* APNN_KERNEL_* */

@@ -52,14 +52,17 @@ def test_gemm_named_entry_golden(G, wb, xb):
 
 # 0 = APNN_PATH_AUTO (the library's own choice: what the named entry points, the networks and the
 # benchmark run), APNN_PATH_VALU, APNN_PATH_MFMA (FP4 operands), APNN_PATH_MFMA_I8
-PATHS = [0, 1, 2, 3]
+# 5 = APNN_PATH_MFMA_XS (FP4 operands expanded by the staging threads)
+PATHS = [0, 1, 2, 3, 5]
 CONV_PATHS = [0, 1, 2, 3, 4]   # 4 = APNN_PATH_MFMA_PATCH (input patch resident in LDS)
+CONV_PATHS_128 = CONV_PATHS + [5]   # shapes whose stored channel count is a multiple of 128
 # (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
 # int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128; int8 convolution
 # 128x128, 64x64, 128x64, 32x32 split-K, 128x256
-GEMM_TILES = [(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)]
+GEMM_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)] +
+              [(5, t) for t in (1, 2, 3, 6)])
 CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
-              [(4, t) for t in range(5)])
+              [(4, t) for t in range(5)] + [(5, t) for t in (1, 2, 3, 7)])
 GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
 CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
 
@@ -170,7 +173,7 @@ def test_conv_named_entry_golden(G, wb, xb):
         assert np.array_equal(G.to_host(outq, np.uint32).reshape(expect.shape), expect)
 
 
-@pytest.mark.parametrize("path", CONV_PATHS)
+@pytest.mark.parametrize("path", CONV_PATHS_128)
 @pytest.mark.parametrize("wb,xb", COMBOS)
 @pytest.mark.parametrize("C,batch", [(128, 1), (256, 1), (512, 1), (128, 16)])
 def test_conv3x3_16x16_sweep(G, wb, xb, C, batch, path):
@@ -234,6 +237,9 @@ def test_conv_general_geometry(G, geom, wb, xb, sym, path):
     expect = O.conv(Wt, X, cwords=cin_pad // 32, sym_w=sym, nthreads=8, **kw)
     got = G.run_conv(Wt, X, cin_pad=cin_pad, sym=sym, path=path, **kw).reshape(expect.shape)
     assert np.array_equal(got, expect)
+    if cin_pad % 128 == 0 and path == 2:      # the expand-while-staging kernel needs 128-bit loads
+        got = G.run_conv(Wt, X, cin_pad=cin_pad, sym=sym, path=5, **kw).reshape(expect.shape)
+        assert np.array_equal(got, expect)
 
 
 @pytest.mark.parametrize("path,tile", CONV_TILES)
@@ -546,10 +552,11 @@ def test_pool_planes_wide_codes(G):
 @pytest.mark.parametrize("mode", ["bn", "lowbits"])
 @pytest.mark.parametrize("pool", [0, 1, 2])
 @pytest.mark.parametrize("xb,ob", [(2, 1), (2, 2), (2, 3), (3, 3), (4, 4), (4, 1), (3, 2), (2, 4)])
-@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (2, 5), (1, None), (4, 0), (4, 1), (4, 4)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (2, 5), (1, None), (4, 0), (4, 1), (4, 4),
+                                       (5, 1), (5, 3), (5, 7)])
 def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
     rng = np.random.default_rng(4000 + 100 * xb + 10 * ob + pool + (tile or 0))
-    batch, H, Wd, C, cout, wb = 2, 6, 10, 64, 96, 1
+    batch, H, Wd, C, cout, wb = 2, 6, 10, (128 if path == 5 else 64), 96, 1
     X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
     Wt = O.random_planes(rng, wb, cout * 9, C // 32)
     kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
@@ -584,7 +591,7 @@ def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
 
 @pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("wb,xb,ob", [(1, 2, 2), (1, 2, 1), (1, 3, 3), (1, 4, 4), (2, 2, 2), (1, 2, 4)])
-@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 6), (2, 5), (3, 2), (1, None)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 6), (2, 5), (3, 2), (1, None), (5, 1), (5, 2), (5, 6)])
 def test_gemm_quantize_pack_all_widths(G, path, tile, wb, xb, ob, sym):
     rng = np.random.default_rng(4100 + 100 * xb + 10 * ob + sym + (tile or 0))
     M, N, K = 80, 192, 384
