@@ -167,6 +167,18 @@ bool fp4_exact(long long kwords, int wb, int xb) {
   return kwords * 32 * ((1LL << wb) - 1) * ((1LL << xb) - 1) < (1LL << 24);
 }
 
+// Whether the quantizing epilogue of the FP4 kernels may compare in fp32: accumulator range (K x weight
+// range x activation range) plus the largest scaled shortcut code stay below 2^24.
+int epilogue_float_ok(const KParams &p, int wb, int xb) {
+  const long long acc = (long long)p.KW * 32 * ((1LL << wb) - 1) * ((1LL << xb) - 1);
+  long long sc = 0;
+  if (p.resid_planes != nullptr) {
+    const long long scale = p.resid_scale < 0 ? -(long long)p.resid_scale : p.resid_scale;
+    sc = scale * ((1LL << p.resid_bits) - 1);
+  }
+  return acc + sc < (1LL << 24) ? 1 : 0;
+}
+
 // Reports a kernel choice instead of launching it (apnn_gemm_plan / apnn_conv_plan).
 int fill_plan(apnn_plan *plan, int path, int kernel, int tile, int tr, int tc, int split_k, const KParams &p,
               int patch_pixels_, bool f4ok) {
@@ -300,6 +312,10 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, b
   // cross-overs on ResNet18 / 16x16 benchmark shapes.
   if (conv) {
     const long long nb32 = ntiles(4);
+    // Long reduction, at least 512 output channels and enough 32x128 tiles for 1.5 work-groups per
+    // compute unit (7x7x512 maps at batch 64, 16x16x512..1024 at batch 16): one activation expansion feeds
+    // four blocks, 11-16 % faster than 32x64 / 128x64 there; with 256 channels or fewer tiles it loses
+    if (vw == 4 && KW >= 64 && rowsB >= 512 && 2 * ntiles(8) >= 3 * cus && nb32 <= 4096) return 8;
     if (KW >= 32 && nb32 <= 256) return 4;   // at most one work-group per compute unit
     if (KW >= 32 && nb32 <= 640) return 5;
     if (KW >= 64 && nb32 <= 3200) return 5;
@@ -380,7 +396,7 @@ int plan_direct(apnn_plan *plan, const KParams &p, bool f4ok) {
 }
 
 int plan_mfma(apnn_plan *plan, bool i8, int tile, const KParams &p, bool f4ok) {
-  const bool split = tile == 4 || tile == 5;
+  const bool split = tile == apnn::MT_32x32_K4 || tile == apnn::MT_32x64_K4 || tile == apnn::MT_32x128_K4;
   return fill_plan(plan, i8 ? APNN_PATH_MFMA_I8 : APNN_PATH_MFMA, i8 ? APNN_KERNEL_MFMA_I8 : APNN_KERNEL_MFMA_FP4, tile,
                    apnn::kMfmaTileA[tile], apnn::kMfmaTileB[tile], split ? 4 : 1, p, 0, f4ok);
 }
@@ -414,6 +430,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   p.planesA = d->wb;
   p.planesB = d->xb;
   const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
+  p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
   if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_XS) && !f4ok) return APNN_EUNSUPPORTED;  // fp32 would round
   if (path == APNN_PATH_MFMA_XS) {
@@ -518,6 +535,7 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
 
   p.planesA = d->xb;
   p.planesB = d->wb;
+  p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;

@@ -70,12 +70,12 @@ APNN_DECL_PATCH(2, 2)
 enum { CORE_I8 = 0, CORE_F4 = 1 };
 
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
-constexpr int kMfmaTileCount = 8;
-constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128};
-constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256};
+constexpr int kMfmaTileCount = 9;
+constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128, 32};
+constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256, 128};
 
 enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
-                MT_256x128 = 6, MT_128x256 = 7, MT_COUNT = 8 };
+                MT_256x128 = 6, MT_128x256 = 7, MT_32x128_K4 = 8, MT_COUNT = 9 };
 
 // Which (core, family, load width, tile, plane counts) combinations are built.  Every kernel
 // instantiation costs seconds of compile time, so only the shapes the dispatcher can choose are kept:
@@ -83,6 +83,7 @@ enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_
 //               128x128, 128x64, 64x64 and the 32x32 split-K tile, with narrower loads 64x64 only
 //   FP4 core  : GEMM: all but 256x256 / 128x256;  convolution: all but 256x256 / 256x128, and only
 //               the two small tiles when the stored channel count allows 32-bit loads only;
+//               plus, for convolution with 128-bit loads, the 32x128 split-K tile;
 //               more than five planes in all (w4a4, w1a8, w2a8): 128x128, 64x64, 32x32 split-K
 //               (convolution with narrower loads: 64x64 only); the int8 core is not built for those.
 constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile, int pa, int pb) {
@@ -96,6 +97,8 @@ constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile, int pa, 
     if (vw != 4) return tile == MT_64x64;
     return tile == MT_128x256 || tile == MT_128x128 || tile == MT_128x64 || tile == MT_64x64 || tile == MT_32x32_K4;
   }
+  // 32x128 split-K: FP4 convolution with 128-bit loads (operands go straight to registers)
+  if (tile == MT_32x128_K4) return conv && vw == 4;
   if (!conv) return tile != MT_256x256 && tile != MT_128x256;
   if (vw == 1) return tile == MT_64x64 || tile == MT_32x32_K4;
   return tile != MT_256x256 && tile != MT_256x128;

@@ -65,6 +65,9 @@ struct KParams {
   int32_t *save_acc;
   const uint32_t *resid_planes;  // packed shortcut codes [resid_bits][rows][rowsB/32]
   int resid_bits, resid_scale;
+  // 1: every value the quantizing epilogue compares (accumulator, correction, scaled shortcut code) is an
+  // integer below 2^24 in magnitude, so the FP4 kernels may do the threshold compare in fp32
+  int epi_float;
   void *out;
   long long out_plane;       // packed output: plane stride in words
 };

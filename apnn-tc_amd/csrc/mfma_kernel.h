@@ -146,11 +146,34 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
 #pragma unroll
   for (int y = 0; y < FB; ++y) cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
 
+  // Float form of the 2-bit threshold compare (FP4 core): the accumulator is acc = raw / 4 in fp32, and
+  // with every operand an integer below 2^24 in magnitude (the host checked: KParams::epi_float)
+  //   v = 2^sh * 4 * acc - correction (+ shortcut)  is one exact fused multiply-add on the accumulator,
+  // compared with the thresholds converted to float (clamped to +-2^24, which no value reaches): four
+  // vector operations per value instead of nine (multiply, convert, shift, subtract, sign flip x2,
+  // compare, select, compare).  Taken when no channel of this wave's tile has the flip flag.
+  float Tf[FB][3];
+  float cnegf[FB];
+  bool fast = false;
+  if constexpr (F4 && !TABLE) {
+    int anyflip = 0;
+#pragma unroll
+    for (int y = 0; y < FB; ++y) {
+      anyflip |= fm[y];
+      cnegf[y] = (float)cneg[y];
+#pragma unroll
+      for (int k = 0; k < 3; ++k) Tf[y][k] = (float)min(max(T[y][k], -(1 << 24)), 1 << 24);
+    }
+    fast = bn && p.epi_float != 0 && p.pool != APNN_POOL_AVG2X2 && __ballot(anyflip != 0) == 0ull;
+  }
+  const float vscale = p.sym ? 8.0f : 4.0f;
+
   // The epilogue mode (thresholds or low bits, pooled or not) is the same for the whole launch: the
   // value loop is instantiated once per mode and entered through one branch, so the per-value code
   // carries no mode tests.
-  auto run = [&](auto bn_c, auto pooled_c) {
+  auto run = [&](auto bn_c, auto pooled_c, auto fast_c) {
     constexpr bool BN = decltype(bn_c)::value, POOLED = decltype(pooled_c)::value;
+    constexpr bool FAST = decltype(fast_c)::value;
     static_for<0, FA>([&](auto xc) {
       constexpr int x = decltype(xc)::value;
       uint32_t park[FB][NPARK];
@@ -162,6 +185,7 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
       static_for<Q0, Q1>([&](auto qc) {
         constexpr int q = decltype(qc)::value;
         int negc[4] = {0, 0, 0, 0};
+        float negcf[4] = {0.f, 0.f, 0.f, 0.f};
         if (CONV) {
           // the row sums were multiplied by the weight range when they were written
           const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
@@ -169,19 +193,30 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
           negc[1] = -rs.y;
           negc[2] = -rs.z;
           negc[3] = -rs.w;
+          if constexpr (FAST) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) negcf[j] = (float)negc[j];
+          }
         }
         static_for<0, FB>([&](auto yc) {
           constexpr int y = decltype(yc)::value;
           int v[4];
+          float u[4];
           static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            int t;
-            if constexpr (F4) {
-              t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+            if constexpr (FAST) {
+              u[j] = __builtin_fmaf((float)acc[x][y][4 * q + j], vscale, CONV ? negcf[j] : cnegf[y]);
+              v[j] = 0;
             } else {
-              t = acc[x][y][4 * q + j];
+              int t;
+              if constexpr (F4) {
+                t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+              } else {
+                t = acc[x][y][4 * q + j];
+              }
+              v[j] = (t << sh) + (CONV ? negc[j] : cneg[y]);
+              u[j] = 0.f;
             }
-            v[j] = (t << sh) + (CONV ? negc[j] : cneg[y]);
           });
           if (!POOLED && shortcut) {
             uint32_t rw[2][4];
@@ -196,12 +231,17 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const int code = (int)(((rw[0][j] >> bitpos) & 1u) | (((rw[1][j] >> bitpos) & 1u) << 1));
-              v[j] += code * p.resid_scale;
+              if constexpr (FAST) {
+                u[j] += (float)(code * p.resid_scale);
+              } else {
+                v[j] += code * p.resid_scale;
+              }
             }
           }
           // one item: value (or code) -> one ballot per output bit, words parked at lanes rlo (lane
           // half 0's row) and rhi (lane half 1's row)
-          auto emit = [&](int val, auto rlo_c, auto rhi_c) {
+          auto emit = [&](auto val, auto rlo_c, auto rhi_c) {
+            using ValT = decltype(val);
             constexpr int rlo = decltype(rlo_c)::value, rhi = decltype(rhi_c)::value;
             auto put = [&](auto slot_c, unsigned long long mask) {
               constexpr int slot = decltype(slot_c)::value;
@@ -215,7 +255,12 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
               reg = write_lane<rhi + 32 * (slot & 1)>(hi, reg);
               park[y][slot >> 1] = (uint32_t)reg;
             };
-            if constexpr (!BN) {
+            if constexpr (std::is_same<ValT, float>::value) {
+              const bool hi1 = val >= Tf[y][1];
+              put(std::integral_constant<int, 1>{}, __ballot(hi1));
+              const float tsel = hi1 ? Tf[y][2] : Tf[y][0];
+              put(std::integral_constant<int, 0>{}, __ballot(val >= tsel));
+            } else if constexpr (!BN) {
               static_for<0, 2 * NPARK>([&](auto bc) {
                 constexpr int b = decltype(bc)::value;
                 if (b < nb) put(bc, __ballot((val >> b) & 1));
@@ -239,7 +284,17 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
             }
           };
           auto flipped = [&](int t) { return (t ^ fm[y]) - fm[y]; };
-          if constexpr (!POOLED) {
+          if constexpr (FAST) {
+            if constexpr (!POOLED) {
+              static_for<0, 4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                emit(u[j], std::integral_constant<int, 8 * q + j>{}, std::integral_constant<int, 8 * q + 4 + j>{});
+              });
+            } else {  // max pooling of codes == code of the maximum (thresholds are monotone, no flip here)
+              emit(fmaxf(fmaxf(u[0], u[1]), fmaxf(u[2], u[3])), std::integral_constant<int, 2 * q>{},
+                   std::integral_constant<int, 2 * q + 1>{});
+            }
+          } else if constexpr (!POOLED) {
             static_for<0, 4>([&](auto jc) {
               constexpr int j = decltype(jc)::value;
               emit(BN ? flipped(v[j]) : (v[j] & lowmask), std::integral_constant<int, 8 * q + j>{},
@@ -291,10 +346,16 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
   };
   using std::false_type;
   using std::true_type;
+  if constexpr (F4 && !TABLE) {
+    if (fast) {
+      if (pooled) run(true_type{}, true_type{}, true_type{}); else run(true_type{}, false_type{}, true_type{});
+      return;
+    }
+  }
   if (bn) {
-    if (pooled) run(true_type{}, true_type{}); else run(true_type{}, false_type{});
+    if (pooled) run(true_type{}, true_type{}, false_type{}); else run(true_type{}, false_type{}, false_type{});
   } else {
-    if (pooled) run(false_type{}, true_type{}); else run(false_type{}, false_type{});
+    if (pooled) run(false_type{}, true_type{}, false_type{}); else run(false_type{}, false_type{}, false_type{});
   }
 }
 
@@ -1070,6 +1131,7 @@ inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t strea
     case MT_128x64: return launch_mfma_if_enabled<CORE, PA, PB, 1, 2, 4, 1, VW, CONV, 4, MT_128x64>(p, stream);
     case MT_32x32_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 1, 1, 1, VW, CONV, 4, MT_32x32_K4>(p, stream);
     case MT_32x64_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 2, 1, 1, VW, CONV, 4, MT_32x64_K4>(p, stream);
+    case MT_32x128_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 4, 1, 1, VW, CONV, 2, MT_32x128_K4>(p, stream);
     case MT_256x128: return launch_mfma_if_enabled<CORE, PA, PB, 4, 2, 2, 2, VW, CONV, 2, MT_256x128>(p, stream);
     case MT_128x256: return launch_mfma_if_enabled<CORE, PA, PB, 2, 4, 2, 2, VW, CONV, 2, MT_128x256>(p, stream);
     default: return hipErrorNotSupported;

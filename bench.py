@@ -145,10 +145,11 @@ def main():
                          "gemm_large, gemm8192 (w1a2 only), conv, nets, resnet18_b8, resnet18_b64, alexnet_b8, "
                          "alexnet_b64, vgg_b8, vgg_b64; crossover (not part of all): every kernel path / tile "
                          "pinned in turn on the shapes where the library's choice changes")
-    ap.add_argument("--path", default="auto", choices=["auto", "valu", "mfma", "mfma_i8"])
+    ap.add_argument("--path", default="auto")
     ap.add_argument("--shape", action="append", default=[],
                     help="extra workload on --path (repeatable; used by the profile commands): "
-                         "gemm:w1a2:M:N:K or conv:w1a2:b16:c1024:int32|fused (3x3 on a 16x16 map)")
+                         "gemm:w1a2:M:N:K or conv:w1a2:b16:c1024:int32|fused[:hN] (3x3 on an NxN map, "
+                         "default 16x16); --path may carry a pinned tile as path/tile, e.g. mfma/5")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also launch one 256 MiB device copy (known traffic) for counter calibration")
     args = ap.parse_args()
@@ -181,7 +182,15 @@ def main():
                                           ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    path = {"auto": A.PATH_AUTO, "valu": A.PATH_VALU, "mfma": A.PATH_MFMA, "mfma_i8": A.PATH_MFMA_I8}[args.path]
+    pname, _, ptile = args.path.partition("/")
+    path = {"auto": A.PATH_AUTO, "valu": A.PATH_VALU, "mfma": A.PATH_MFMA, "mfma_i8": A.PATH_MFMA_I8,
+            "patch": A.PATH_MFMA_PATCH, "mfma_xs": A.PATH_MFMA_XS}[pname]
+    if ptile:
+        path |= (int(ptile) + 1) << 8
+    # the headline and the standard extra workloads run on the plain path; a pinned tile or a
+    # convolution-only / GEMM-subset path applies to the --shape workloads only
+    plain = not ptile and pname in ("auto", "valu", "mfma", "mfma_i8")
+    cur = {"path": path if plain else A.PATH_AUTO}
 
     def make_inputs(M, N, K, wb, xb):
         W = O.random_planes(np.random.default_rng(0x5EED0001), wb, M, K // 32)
@@ -193,7 +202,7 @@ def main():
         dW, dX = G.to_dev(W), G.to_dev(X)
         out = G.dev_empty_i32(M * N, fill=-7)
         d = A.GemmDesc(W=dW.data_ptr(), X=dX.data_ptr(), D=out.data_ptr(), M=M, N=N, K=K, wb=wb, xb=xb,
-                       weight_mode=sym, path=path)
+                       weight_mode=sym, path=cur["path"])
         ev, wall = ctypes.c_float(), ctypes.c_double()
         torch.cuda.synchronize()
         if graph:
@@ -282,12 +291,12 @@ def main():
 
     conv_ref_cache = {}
 
-    def time_conv(batch, C, w_, a_, fused, warmup, iters):
+    def time_conv(batch, C, w_, a_, fused, warmup, iters, H=16):
         """3x3, stride 1, stored halo, 16x16 feature map, Cin = Cout = C (the reference's conv benchmark,
         APNN-TC-lib/bmmaTensorCoreGemm/src/51_conv_w1a2_small.cu:478-512, with a batch dimension).  Every
         row is checked against the oracle: the int32 output as is, the fused output against the oracle's
         threshold quantizer + packer applied to the oracle convolution."""
-        H = Wd = 16
+        Wd = H
         rng = np.random.default_rng(0x5EED0003)
         X = O.random_planes(rng, a_, batch * (H + 2) * (Wd + 2), C // 32)
         # the halo ring holds zeros, as the reference's padded input does
@@ -295,7 +304,7 @@ def main():
         Xv[:, :, 0], Xv[:, :, -1], Xv[:, :, :, 0], Xv[:, :, :, -1] = 0, 0, 0, 0
         Wt = O.random_planes(rng, w_, C * 9, C // 32)
         dW, dX = G.to_dev(Wt), G.to_dev(X)
-        key = (batch, C, w_, a_)
+        key = (batch, C, w_, a_, H)
         if key not in conv_ref_cache:
             conv_ref_cache.clear()      # rows of one shape are adjacent: keep one reference at a time
             conv_ref_cache[key] = O.conv(Wt, X, batch=batch, H=H, W=Wd, cwords=C // 32, cout=C, R=3, S=3, stride=1,
@@ -314,7 +323,7 @@ def main():
             nbytes = (a_ * batch * H * Wd * C + w_ * 9 * C * C) // 8 + 4 * batch * H * Wd * C
         d = A.ConvDesc(W=dW.data_ptr(), X=dX.data_ptr(), O=out.data_ptr(), batch=batch, H=H, Wd=Wd, cin_pad=C, COUT=C,
                        R=3, S=3, stride=1, pad=1, halo=1, wb=w_, xb=a_, weight_mode=A.WEIGHT_UNSIGNED, epi=E,
-                       path=path)
+                       path=cur["path"])
         ev, wall = ctypes.c_float(), ctypes.c_double()
         if batch == 1:
             A.check(benchlib.apnn_bench_conv_graph(ctypes.byref(d), warmup, iters, GRAPH_BATCH, ctypes.byref(ev),
@@ -352,6 +361,27 @@ def main():
                                "frac_hbm_peak": round(nb / (t["event_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
                                "verified": t["verified"]})
             large = (2048, 4096, 8192) if on("gemm_large") else ((8192,) if (w_, a_) == (1, 2) and on("gemm8192") else ())
+            for n in large if (w_, a_) == (1, 2) else ():
+                # the same GEMM with the low a bits packed (apmm_w1a2_decompose): no 4*M*N-byte int32 store
+                W, X = make_inputs(n, n, n, w_, a_)
+                dW, dX = G.to_dev(W), G.to_dev(X)
+                outp = G.dev_empty_i32(a_ * n * n // 32, fill=-7)
+                dd = A.GemmDesc(W=dW.data_ptr(), X=dX.data_ptr(), D=outp.data_ptr(), M=n, N=n, K=n, wb=w_, xb=a_,
+                                epi=G.epilogue(mode=A.EPI_LOWBITS, out_bits=a_), path=cur["path"])
+                ev, wall = ctypes.c_float(), ctypes.c_double()
+                iters = {2048: 20, 4096: 10, 8192: 3}[n]
+                A.check(benchlib.apnn_bench_gemm(ctypes.byref(dd), 2, iters, stream, ctypes.byref(ev), ctypes.byref(wall)),
+                        "apnn_bench_gemm(packed)")
+                torch.cuda.synchronize()
+                gotp = G.to_host(outp, np.uint32).reshape(a_, n, n // 32)
+                okp = True
+                for m in (0, n // 2 + 1, n - 1):
+                    ref = O.gemm_rows(W, X, n, n, n, w_, a_, m, m + 1, nthreads=os.cpu_count() or 1)
+                    okp = okp and bool(np.array_equal(gotp[:, m], O.lowbits_pack(ref, 1, n, a_)[:, 0]))
+                tt = 2.0 * n ** 3 / (ev.value / iters * 1e-3) / 1e12
+                shapes.append({"shape": "w%da%d M=N=K=%d low-bit packed out" % (w_, a_, n), "ms": round(ev.value / iters, 4),
+                               "tops": round(tt, 2), "frac_fp4_mfma_peak": round(tt / FP4_MFMA_PEAK_TOPS, 4),
+                               "verified": okp})
             for n in large:
                 iters = {2048: 20, 4096: 10, 8192: 3}[n]
                 vrows = sorted(set([0, n - 1] + [int(v) for v in np.random.default_rng(n).integers(0, n, 14)]))
@@ -385,7 +415,7 @@ def main():
                 if not on("nets", "%s_b%d" % (nm, batch)):
                     continue
                 NL = A.nn_lib()
-                net = NL.apnn_net_create(kind, batch, 1, path)
+                net = NL.apnn_net_create(kind, batch, 1, cur["path"])
                 assert net, "network construction failed"
                 img = torch.randint(0, 256, (batch, 224, 224, 3), dtype=torch.uint8, device="cuda")
                 lg = torch.empty((batch, 1000), dtype=torch.float32, device="cuda")
@@ -420,6 +450,7 @@ def main():
                 NL.apnn_net_destroy(net)
         if nets:
             extra["networks"] = nets
+    cur["path"] = path
     for spec in args.shape:
         f = spec.split(":")
         w_, a_ = int(f[1][1]), int(f[1][3])
@@ -434,7 +465,8 @@ def main():
                                                       "tops": round(tt, 2), "verified": t["verified"]})
         else:
             bt, Cc = int(f[2][1:]), int(f[3][1:])
-            t = time_conv(bt, Cc, w_, a_, f[4] == "fused", 200 if bt == 1 else 10, 1000 if bt == 1 else 50)
+            Hm = int(f[5][1:]) if len(f) > 5 else 16
+            t = time_conv(bt, Cc, w_, a_, f[4] == "fused", 200 if bt == 1 else 10, 1000 if bt == 1 else 50, H=Hm)
             t.update(shape=spec, path=args.path)
             extra.setdefault("requested", []).append(t)
     if "crossover" in want:

@@ -57,11 +57,11 @@ PATHS = [0, 1, 2, 3, 5]
 CONV_PATHS = [0, 1, 2, 3, 4]   # 4 = APNN_PATH_MFMA_PATCH (input patch resident in LDS)
 CONV_PATHS_128 = CONV_PATHS + [5]   # shapes whose stored channel count is a multiple of 128
 # (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
-# int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128; int8 convolution
+# int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128 (8 = 32x128 split-K); int8 convolution
 # 128x128, 64x64, 128x64, 32x32 split-K, 128x256
 GEMM_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)] +
               [(5, t) for t in (1, 2, 3, 6)])
-CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
+CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7, 8)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
               [(4, t) for t in range(5)] + [(5, t) for t in (1, 2, 3, 7)])
 GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
 CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
@@ -552,11 +552,11 @@ def test_pool_planes_wide_codes(G):
 @pytest.mark.parametrize("mode", ["bn", "lowbits"])
 @pytest.mark.parametrize("pool", [0, 1, 2])
 @pytest.mark.parametrize("xb,ob", [(2, 1), (2, 2), (2, 3), (3, 3), (4, 4), (4, 1), (3, 2), (2, 4)])
-@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (2, 5), (1, None), (4, 0), (4, 1), (4, 4),
-                                       (5, 1), (5, 3), (5, 7)])
+@pytest.mark.parametrize("path,tile", [(2, 1), (2, 2), (2, 3), (2, 7), (2, 4), (2, 5), (2, 8), (1, None), (4, 0), (4, 1),
+                                       (4, 4), (5, 1), (5, 3), (5, 7)])
 def test_conv_quantize_pack_all_widths(G, path, tile, xb, ob, pool, mode):
     rng = np.random.default_rng(4000 + 100 * xb + 10 * ob + pool + (tile or 0))
-    batch, H, Wd, C, cout, wb = 2, 6, 10, (128 if path == 5 else 64), 96, 1
+    batch, H, Wd, C, cout, wb = 2, 6, 10, (128 if path == 5 or tile == 8 else 64), 96, 1
     X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
     Wt = O.random_planes(rng, wb, cout * 9, C // 32)
     kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
