@@ -47,18 +47,31 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 // FP4 operand for digit D (planes 2D and, if present, 2D+1) of a P-plane row word: nibble c of
 // result word t is the digit of element 4c + t.
+// One plane: shift and mask per result word, 7 operations.  Two planes: the planes are first merged
+// into two words of sixteen 2-bit digits (even elements, odd elements; one bit-field insert each), and
+// every result word is a shift and a mask of one of those, 10 operations instead of 14 for separate
+// shifts and masks of both planes.
 template <int P, int D>
 __device__ __forceinline__ v8i expand_fp4(const uint32_t (&w)[P]) {
   v8i out = {0, 0, 0, 0, 0, 0, 0, 0};
   const uint32_t x0 = w[2 * D];
+  if constexpr (2 * D + 1 < P) {
+    const uint32_t x1 = w[2 * D + 1];
+    constexpr uint32_t EVEN = 0x55555555u;
+    // digit of element 2i at bits 2i, 2i+1
+    uint32_t qe = (x0 & EVEN) | ((x1 << 1) & ~EVEN);
+    uint32_t qo = ((x0 >> 1) & EVEN) | (x1 & ~EVEN);
+    // keep the merged words: without this the optimizer distributes the masks below over the two
+    // planes again and emits the 14-operation form
+    asm("" : "+v"(qe));
+    asm("" : "+v"(qo));
+    out[0] = (int)(qe & 0x33333333u);
+    out[1] = (int)(qo & 0x33333333u);
+    out[2] = (int)((qe >> 2) & 0x33333333u);
+    out[3] = (int)((qo >> 2) & 0x33333333u);
+  } else {
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    uint32_t word = (x0 >> t) & 0x11111111u;
-    if constexpr (2 * D + 1 < P) {
-      const uint32_t x1 = w[2 * D + 1];
-      word |= (t == 0 ? (x1 << 1) : (x1 >> (t - 1))) & 0x22222222u;
-    }
-    out[t] = (int)word;
+    for (int t = 0; t < 4; ++t) out[t] = (int)((x0 >> t) & 0x11111111u);
   }
   return out;
 }
@@ -359,6 +372,62 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
   }
 }
 
+// int32 output straight from the accumulators.  Register r of a 32x32 block is row 8*(r/4) + 4*g + r%4,
+// column li, and the output is row-major with the column index fastest, so one store instruction of the
+// wave writes two full 128-byte rows of the block (one per lane half): no LDS round trip, two vector
+// operations per value (scale, convert) and one address update per output row.  lds[0 .. FA*32) holds
+// the activation row sums times the weight range (convolution with symmetric weights; unused otherwise).
+template <bool F4, int FA, int FB, bool CONV, class AccT>
+__device__ __forceinline__ void store_int32_direct(const KParams &p, AccT (&acc)[FA][FB],
+                                                   const int (&ssum)[CONV ? FA : FB], const uint32_t *lds,
+                                                   int rbase, int cbase, int lane) {
+  const int li = lane & 31, g = lane >> 5;
+  const int sh = p.sym ? 1 : 0;
+  const int wmax = p.sym ? p.wmax : 0;
+  const int *rowsum = reinterpret_cast<const int *>(lds);
+  int cneg[FB];
+#pragma unroll
+  for (int y = 0; y < FB; ++y) cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
+  int *out = reinterpret_cast<int *>(p.out);
+  const long long pitch = p.rowsB;
+  const bool full = rbase + FA * 32 <= p.rowsA && cbase + FB * 32 <= p.rowsB;  // same for the whole wave
+  auto run = [&](auto full_c) {
+    constexpr bool FULL = decltype(full_c)::value;
+    int *rowp = out + (long long)(rbase + 4 * g) * pitch + cbase + li;
+    static_for<0, FA>([&](auto xc) {
+      constexpr int x = decltype(xc)::value;
+      static_for<0, 4>([&](auto qc) {
+        constexpr int q = decltype(qc)::value;
+        int negc[4] = {0, 0, 0, 0};
+        if (CONV && p.sym) {
+          const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
+          negc[0] = -rs.x;
+          negc[1] = -rs.y;
+          negc[2] = -rs.z;
+          negc[3] = -rs.w;
+        }
+        static_for<0, 4>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          int *dst = rowp + (long long)(x * 32 + 8 * q + j) * pitch;
+          const bool row_ok = FULL || rbase + x * 32 + 8 * q + 4 * g + j < p.rowsA;
+          static_for<0, FB>([&](auto yc) {
+            constexpr int y = decltype(yc)::value;
+            int t;
+            if constexpr (F4) {
+              t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+            } else {
+              t = acc[x][y][4 * q + j];
+            }
+            const int v = (t << sh) + (CONV ? negc[j] : cneg[y]);
+            if (FULL || (row_ok && cbase + y * 32 + li < p.rowsB)) dst[y * 32] = v;
+          });
+        });
+      });
+    });
+  };
+  if (full) run(std::true_type{}); else run(std::false_type{});
+}
+
 // Output stage of one wave for a 32-row slab of its tile, staged in LDS as slab[32][NCOLS + 1]
 // (row-major, so the 64 lanes walk 64 consecutive output channels).  rowsum / colsum hold the
 // activation sums for the symmetric-weight correction (rows for convolution, columns for the GEMM
@@ -577,6 +646,17 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
     }
   }
   if constexpr (KS == 1) {
+    if (p.epi == APNN_EPI_INT32) {
+      uint32_t *area = smem + wave * SLAB_WORDS;
+      if (CONV && p.sym) {
+        if (g == 0) {
+#pragma unroll
+          for (int x = 0; x < FA; ++x) area[x * 32 + li] = (uint32_t)(p.wmax * ssum[CONV ? x : 0]);
+        }
+      }
+      store_int32_direct<F4, FA, FB, CONV>(p, acc, ssum, area, a0 + wa * FA * 32, b0 + wb * FB * 32, lane);
+      return;
+    }
     if (direct) {
       uint32_t *area = smem + wave * SLAB_WORDS;
       if (CONV && g == 0) {
@@ -975,7 +1055,9 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   // the last k-step of chunk ch).  Global loads run two chunks ahead, LDS holds two chunks.
   constexpr int NKS = KC / WPS;  // k-steps per chunk
   constexpr int N_MFMA = FA * FB * DA * DB;
-  constexpr int N_VALU = (F4 ? 7 : 8) * (FA * PA + FB * PB) + FS * PS;
+  // expansion cost per row word: FP4 10 operations per plane pair + 7 for an odd plane, int8 8 per plane
+  constexpr int XA = F4 ? 10 * (PA / 2) + 7 * (PA % 2) : 8 * PA, XB = F4 ? 10 * (PB / 2) + 7 * (PB % 2) : 8 * PB;
+  constexpr int N_VALU = FA * XA + FB * XB + FS * PS;
   constexpr int VALU_PER_MFMA = (N_VALU + N_MFMA - 1) / N_MFMA;
 
   auto direct_loop = [&]() {
