@@ -278,7 +278,8 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, bool wide = false) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3) {
+  const bool wide = planes > 5;
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
@@ -324,9 +325,11 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, b
   if (rowsB > 64) {
     const int big = conv ? 7 : 6;
     if (ntiles(big) >= cus && fill(big) >= 0.8) return big;
-    // 128x128 wants more than one work-group per compute unit (measured: with exactly one, the 128x64
-    // tile's two work-groups per compute unit are 4-9 % faster, GEMM 2048^3 and convolution 4096 x 1024)
-    if (2 * ntiles(1) >= 3 * cus && fill(1) >= 0.8) return 1;
+    // 128x128 wants more than one work-group per compute unit (measured with three planes in all: with
+    // exactly one, the 128x64 tile's two work-groups per compute unit are 3-9 % faster, GEMM 2048^3 and
+    // convolution 4096 x 1024; with five planes the larger tile's lower expansion cost per matrix
+    // instruction wins by 11 %, w1a4 2048^3)
+    if ((planes > 3 ? ntiles(1) >= cus : 2 * ntiles(1) >= 3 * cus) && fill(1) >= 0.8) return 1;
     if (ntiles(3) >= cus && fill(3) >= 0.8) return 3;
     if (ntiles(1) >= cus && fill(1) >= 0.8) return 1;
   }
@@ -342,7 +345,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, b
 
 int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB > 5);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;

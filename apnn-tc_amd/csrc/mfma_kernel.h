@@ -9,8 +9,8 @@
 //           2-bit digits (plane pairs); digit pair (da, db) is one instruction per 32x32 block and
 //           64 k -- at the same issue cost as the int8 instruction, so twice its rate -- with the
 //           weight 4^(da+db) applied by the instruction's E8M0 block scale.  Products are multiples
-//           of 1/4 and partial sums stay far below 2^22, so the fp32 accumulators are exact and the
-//           result is acc * 4.
+//           of 1/4 and the host only launches this core while K * (2^w - 1) * (2^a - 1) < 2^24, so the
+//           fp32 accumulators are exact and the result is acc * 4.
 //
 // Work-group = 4 waves arranged WA x WB, each wave owning an (FA*32) x (FB*32) output tile
 // (FA*FB accumulator blocks of 16 registers).  The *packed* planes are staged through LDS
@@ -19,15 +19,16 @@
 //   lane (i, g) of a wave supplies row i and the 16 k-positions { 8c + 4g + t : c,t < 4 } of the
 //   word -- the same positions for both operands, so the contraction pairs bit k with bit k as the
 //   reference does (APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:364-369).
-//   ys_p = rotr(word_p, 4g - p);  byte-word t = OR_p ((ys_p >> t) & (0x01010101 << p))
-// i.e. 8 VALU operations per plane for 16 int8 operands.
+//   CORE_I8: ys_p = rotr(word_p, 4g - p);  byte-word t = OR_p ((ys_p >> t) & (0x01010101 << p)),
+//   i.e. 8 VALU operations per plane for 16 int8 operands; CORE_F4: see expand_fp4.
 //
 // Symmetric (+-) weights use the closed form  2*raw - wmax * (activation row sum); the row sums
 // come from popcounts of the packed words the wave already holds.
 //
-// The epilogue passes each wave's tile through an LDS slab, 32 rows at a time, to turn the
-// matrix-core register layout into row-major order: stores are contiguous, and 64 consecutive
-// channels sit in the 64 lanes so that one ballot per output bit yields two MSB-first words.
+// Output: int32 results and codes of up to two bits (four where the waves tile the output) leave
+// straight from the accumulator registers (store_int32_direct, direct_epilogue); int32 residuals, saved
+// accumulators and wider codes pass each wave's tile through an LDS slab, 32 rows at a time, which turns
+// the matrix-core register layout into row-major order.
 #pragma once
 #include <hip/hip_runtime.h>
 
