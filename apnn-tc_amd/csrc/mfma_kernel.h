@@ -387,8 +387,15 @@ __device__ __forceinline__ void store_int32_direct(const KParams &p, AccT (&acc)
   const int wmax = p.sym ? p.wmax : 0;
   const int *rowsum = reinterpret_cast<const int *>(lds);
   int cneg[FB];
+  float cnegf[FB];
 #pragma unroll
-  for (int y = 0; y < FB; ++y) cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
+  for (int y = 0; y < FB; ++y) {
+    cneg[y] = CONV ? 0 : -wmax * ssum[CONV ? 0 : y];
+    cnegf[y] = (float)cneg[y];
+  }
+  // FP4 core: value = acc * 4 * 2^sym - correction as one fused multiply-add in fp32 and one conversion
+  // (the host launches this core only while every such value is an integer below 2^24, so both are exact)
+  const float vscale = p.sym ? 8.0f : 4.0f;
   int *out = reinterpret_cast<int *>(p.out);
   const long long pitch = p.rowsB;
   const bool full = rbase + FA * 32 <= p.rowsA && cbase + FB * 32 <= p.rowsB;  // same for the whole wave
@@ -400,12 +407,15 @@ __device__ __forceinline__ void store_int32_direct(const KParams &p, AccT (&acc)
       static_for<0, 4>([&](auto qc) {
         constexpr int q = decltype(qc)::value;
         int negc[4] = {0, 0, 0, 0};
+        float negcf[4] = {0.f, 0.f, 0.f, 0.f};
         if (CONV && p.sym) {
           const int4 rs = *reinterpret_cast<const int4 *>(rowsum + x * 32 + 8 * q + 4 * g);
           negc[0] = -rs.x;
           negc[1] = -rs.y;
           negc[2] = -rs.z;
           negc[3] = -rs.w;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) negcf[j] = (float)negc[j];
         }
         static_for<0, 4>([&](auto jc) {
           constexpr int j = decltype(jc)::value;
@@ -413,13 +423,12 @@ __device__ __forceinline__ void store_int32_direct(const KParams &p, AccT (&acc)
           const bool row_ok = FULL || rbase + x * 32 + 8 * q + 4 * g + j < p.rowsA;
           static_for<0, FB>([&](auto yc) {
             constexpr int y = decltype(yc)::value;
-            int t;
+            int v;
             if constexpr (F4) {
-              t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+              v = (int)__builtin_fmaf((float)acc[x][y][4 * q + j], vscale, CONV ? negcf[j] : cnegf[y]);
             } else {
-              t = acc[x][y][4 * q + j];
+              v = (acc[x][y][4 * q + j] << sh) + (CONV ? negc[j] : cneg[y]);
             }
-            const int v = (t << sh) + (CONV ? negc[j] : cneg[y]);
             if (FULL || (row_ok && cbase + y * 32 + li < p.rowsB)) dst[y * 32] = v;
           });
         });
