@@ -132,7 +132,7 @@ template <bool F4, int FA, int FB, bool CONV, bool TABLE, int Q0 = 0, int Q1 = 4
 __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA][FB],
                                                 const int (&ssum)[CONV ? FA : FB], uint32_t *lds, int rbase,
                                                 int cbase, int lane, const int (&T)[FB][3], const int (&fm)[FB],
-                                                bool shortcut) {
+                                                bool shortcut, const int *shared_table = nullptr) {
   constexpr int NCOLS = FB * 32;
   constexpr int NPARK = TABLE ? 2 : 1;
   const int li = lane & 31, g = lane >> 5;
@@ -146,14 +146,16 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
   const int w32 = p.rowsB >> 5;
   const int *rowsum = reinterpret_cast<const int *>(lds);
   const uint32_t *res = lds + FA * 32;
-  int *tl = reinterpret_cast<int *>(lds + FA * 32 + FA * 64 * FB);
-  if (TABLE && bn) {
+  // threshold table [k][NCOLS]: this wave's own copy, filled here, or one the caller filled for the tile
+  int *own_table = reinterpret_cast<int *>(lds + FA * 32 + FA * 64 * FB);
+  const int *tl = shared_table != nullptr ? shared_table : own_table;
+  if (TABLE && bn && shared_table == nullptr) {
     const int nt = (1 << nb) - 1;
 #pragma unroll
     for (int y = 0; y < FB; ++y) {
       const int gcol = cbase + y * 32 + li;
       if (gcol < p.rowsB)
-        for (int k = g; k < nt; k += 2) tl[k * NCOLS + y * 32 + li] = p.thr[(long long)gcol * nt + k];
+        for (int k = g; k < nt; k += 2) own_table[k * NCOLS + y * 32 + li] = p.thr[(long long)gcol * nt + k];
     }
   }
   int cneg[FB];  // GEMM entry points: the correction depends on the column only
@@ -549,7 +551,7 @@ __device__ __forceinline__ void epi_load(const KParams &p, int rbase, int cbase,
 // registers to spare for values that are idle during the K loop).
 template <int KS, int DIRECT_BITS, bool LAZY, int FA, int FB>
 __device__ __forceinline__ void epi_prefetch(const KParams &p, int rbase, int cbase, int lane, EpiOperands<FA, FB> &eo) {
-  eo.direct = p.epi != APNN_EPI_INT32 && p.out_bits <= (KS == 1 ? DIRECT_BITS : 2) && p.resid == nullptr &&
+  eo.direct = p.epi != APNN_EPI_INT32 && p.out_bits <= DIRECT_BITS && p.resid == nullptr &&
               p.save_acc == nullptr && (p.resid_planes == nullptr || p.resid_bits <= 2);
   eo.q0 = ChannelQuant{};
   eo.q1 = ChannelQuant{};
@@ -592,10 +594,24 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
       constexpr int PART_WORDS = KS * FB * 4 * 64 * 4;
       constexpr int SUM_WORDS = KS * FB * 32;
       constexpr int AREA_WORDS = 32 + 64 * FB;
-      static_assert(PART_WORDS + SUM_WORDS + KS * AREA_WORDS <= KS * SLAB_WORDS, "fits the slab area");
+      // codes of three or four bits: one threshold table [15][NCOLS] for the tile, behind the waves' areas
+      // (the four waves finish different rows of the same columns)
+      constexpr int TABLE_WORDS = DIRECT_BITS > 2 ? 15 * NCOLS : 0;
+      static_assert(PART_WORDS + SUM_WORDS + KS * AREA_WORDS + TABLE_WORDS <= KS * SLAB_WORDS + TABLE_WORDS,
+                    "fits the slab area");
       Acc4 *part = reinterpret_cast<Acc4 *>(smem);
       int *sums = reinterpret_cast<int *>(smem) + PART_WORDS;
       uint32_t *area = smem + PART_WORDS + SUM_WORDS + wave * AREA_WORDS;
+      int *table = reinterpret_cast<int *>(smem) + KS * SLAB_WORDS;
+      const bool use_table = DIRECT_BITS > 2 && p.out_bits > 2;
+      if (DIRECT_BITS > 2 && use_table && p.epi == APNN_EPI_BN) {
+        const int nt = (1 << p.out_bits) - 1;
+        for (int i = threadIdx.x; i < nt * NCOLS; i += 256) {
+          const int k = i / NCOLS, c = i - k * NCOLS;
+          const int gcol = b0 + c;
+          table[i] = gcol < p.rowsB ? p.thr[(long long)gcol * nt + k] : 0;
+        }
+      }
       static_for<0, FB>([&](auto yc) {
         constexpr int y = decltype(yc)::value;
         static_for<0, 4>([&](auto qc) {
@@ -643,6 +659,13 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
           accr[0][y][4 * q + 2] = t.z;
           accr[0][y][4 * q + 3] = t.w;
         });
+        if constexpr (DIRECT_BITS > 2) {
+          if (use_table) {
+            direct_epilogue<F4, 1, FB, CONV, true, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm,
+                                                             res_prefetched, table);
+            return;
+          }
+        }
         direct_epilogue<F4, 1, FB, CONV, false, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm, res_prefetched);
       };
       static_assert(KS == 4, "one register quad per wave");
@@ -1176,7 +1199,10 @@ constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int W
   const size_t stage = core == CORE_F4 && WA * WB == 1 && vw == 4
                            ? 0
                            : 2ull * ((size_t)PA * WA * FA * 32 + (size_t)PB * WB * FB * 32) * ld * sizeof(uint32_t);
-  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int);
+  // split-K tiles whose activations have three or more planes quantize codes of up to four bits from
+  // registers and keep one threshold table [15][FB * 32] behind the output stage's area
+  const size_t table = (WA * WB == 1 && (conv ? PA : PB) >= 3) ? 15ull * FB * 32 * sizeof(int) : 0;
+  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int) + table;
   return stage > slab ? stage : slab;
 }
 
