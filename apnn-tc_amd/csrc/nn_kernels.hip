@@ -338,8 +338,11 @@ __device__ __forceinline__ int write_lane_n(int val, int old) {
 // The epilogue is the compare-is-ballot scheme of the matrix-core kernels: per accumulator register
 // two compares and a select give both bit-plane masks of two output pixels.
 // Requires C <= 4, (W*C) % 4 == 0, X 4-byte aligned, bits <= 2, COUT % 32 == 0.
-template <int NKS>
-__global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+// NWAV waves per work-group share one filter block in LDS (each wave has its own patch and walks its
+// own pixel groups): eight waves where the filter block is large, so that its LDS cost per wave halves
+// and four waves per SIMD stay resident.
+template <int NKS, int NSLOT, int NWAV>
+__global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                            const int32_t *__restrict__ thr,
                                                            uint32_t *__restrict__ planes, int B, int H, int W, int C,
                                                            int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
@@ -363,12 +366,12 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   // all their byte loads are issued before the first LDS store, so the block costs one or two memory
   // round trips instead of one per task.
   const int ntasks = 64 * nks * 2;
-  for (int t0 = 0; t0 < ntasks; t0 += 4 * 256) {
+  for (int t0 = 0; t0 < ntasks; t0 += 4 * 64 * NWAV) {
     uint32_t w[4][4];
     int dst_off[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int task = t0 + u * 256 + tid;
+      const int task = t0 + u * 64 * NWAV + tid;
       const int col = (int)quot((uint32_t)task, (uint32_t)(nks * 2), magic_nh2), hh = task - col * (nks * 2);
       const int r = (int)quot((uint32_t)hh, (uint32_t)HPR, magic_hpr), hq = hh - r * HPR;
       dst_off[u] = col * KPL + hh * 16;
@@ -400,7 +403,7 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int task = t0 + u * 256 + tid;
+      const int task = t0 + u * 64 * NWAV + tid;
       if (task < ntasks) *reinterpret_cast<uint4 *>(wl + dst_off[u]) = make_uint4(w[u][0], w[u][1], w[u][2], w[u][3]);
     }
   }
@@ -444,8 +447,8 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
 
   // Patch element idx = slot * 64 + lane is dword d of row segment r, the same for every group:
   // (r, d) is decoded once.  The raw dwords of the next group are requested before the current
-  // group is computed (patches of up to 512 dwords; larger ones are staged in place).
-  constexpr int NSLOT = 8;
+  // group is computed (patches of up to 64 * NSLOT dwords: NSLOT = 8 covers a 7x7 stride-2 filter on
+  // three channels, 18 an 11x11 stride-4 one; larger patches are staged in place, chunk by chunk).
   const bool prefetch = npatch <= 64 * NSLOT;
   int rd[NSLOT];
 #pragma unroll
@@ -496,8 +499,8 @@ __global__ __launch_bounds__(256) void conv_i8_rows_kernel(const uint8_t *__rest
   };
 
   // (the launcher keeps the number of groups below 2^31: 32-bit index arithmetic)
-  const uint32_t gstep = gridDim.x * 4u, ng = (uint32_t)ngroups;
-  uint32_t group = blockIdx.x * 4u + (uint32_t)wave;
+  const uint32_t gstep = gridDim.x * (uint32_t)NWAV, ng = (uint32_t)ngroups;
+  uint32_t group = blockIdx.x * (uint32_t)NWAV + (uint32_t)wave;
   if (prefetch && group < ng) request(group, 0);
   for (; group < ng; group += gstep) {
     const uint32_t trow = quot(group, (uint32_t)gpr, magic_gpr);
@@ -873,19 +876,36 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
     const int NDW = (3 + (31 * stride + S) * C + 3) / 4;
     const int need = (3 + 31 * stride * C + 16 * (HPR - 1) + 20 + 3) / 4;
     const int PWD = (need > NDW ? need : NDW) | 1;  // odd pitch
-    const size_t lds = (size_t)64 * (nks * 32 + 16) + 4 * (size_t)R * PWD * 4;
-    if (lds <= 64 * 1024) {
+    // slots of image dwords a lane keeps in flight: 8 where that covers the patch, else 18 together with
+    // eight waves per work-group (large filters: 11x11)
+    const bool wide_patch = R * NDW > 64 * 8;
+    const int nwav = wide_patch ? 8 : 4;
+    const size_t lds = (size_t)64 * (nks * 32 + 16) + (size_t)nwav * R * PWD * 4;
+    if (lds <= (wide_patch ? 80 * 1024 : 64 * 1024)) {
       // persistent grid: exactly as many work-groups as the device holds at once
       // Filter block in registers (two work-groups per compute unit fit) while one or two rounds of
       // work-groups cover all pixel groups; beyond that the variant that re-reads the filter from LDS
       // wins through its higher occupancy (four per compute unit).
-      const bool wreg = nks == 7 && grid.x <= 1024;
-      auto kern = wreg ? conv_i8_rows_kernel<7> : conv_i8_rows_kernel<0>;
+      const bool wreg = nks == 7 && grid.x <= 1024 && !wide_patch;
+      auto kern = wreg ? conv_i8_rows_kernel<7, 8, 4>
+                       : (wide_patch ? conv_i8_rows_kernel<0, 18, 8> : conv_i8_rows_kernel<0, 8, 4>);
+      if (wide_patch) {
+        grid.x = (unsigned)((groups + 7) / 8);
+        if (lds > 64 * 1024) {
+          static bool raised = false;
+          if (!raised) {
+            const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+            if (e0 != hipSuccess) return e0;
+            raised = true;
+          }
+        }
+      }
       int per_cu = 0, cus = 0, dev = 0;
       hipError_t e = hipGetDevice(&dev);
       if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
       if (e == hipSuccess)
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern), 256, lds);
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern), 64 * nwav, lds);
       if (e != hipSuccess) return e;
       unsigned resident = (unsigned)(per_cu > 0 ? per_cu : 1) * (unsigned)(cus > 0 ? cus : 256);
       const unsigned slices = grid.y > 0 ? grid.y : 1;
@@ -899,17 +919,13 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
         return (d >= 2 && ngr * d < (1ull << 32)) ? (uint32_t)(((1ull << 32) + d - 1) / d) : 0u;
       };
       const uint32_t mg = magic(gpr), mh = magic((unsigned long long)Ho);
-      // small dividends (patch slots below 512, filter tasks below 2^16): always exact
+      // small dividends (patch slots below 1152, filter tasks below 2^16): always exact
       auto small_magic = [](int d) { return d >= 2 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
       const uint32_t mn = small_magic(NDW), mt = small_magic(nks * 2), mp = small_magic(HPR);
       // the filter array as aligned dwords: base 4-byte aligned and a whole number of dwords long
       const int wt_dwords = (reinterpret_cast<uintptr_t>(Wt) & 3u) == 0 && ((long long)COUT * R * S * C) % 4 == 0;
-      if (wreg)
-        hipLaunchKernelGGL(conv_i8_rows_kernel<7>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh, mn, mt, mp, wt_dwords);
-      else
-        hipLaunchKernelGGL(conv_i8_rows_kernel<0>, g2, dim3(256), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S,
-                           stride, pad, Ho, Wo, bits, xm, HPR, NDW, PWD, mg, mh, mn, mt, mp, wt_dwords);
+      hipLaunchKernelGGL(kern, g2, dim3(64 * nwav), lds, s, Xu, Wt, thr, planes, B, H, W, C, COUT, R, S, stride, pad, Ho,
+                         Wo, bits, xm, HPR, NDW, PWD, mg, mh, mn, mt, mp, wt_dwords);
       return hipGetLastError();
     }
   }
