@@ -356,7 +356,9 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
   const int nks = (NH + 1) / 2;
   const int KB = nks * 32, KPL = KB + 16;
   int8_t *wl = reinterpret_cast<int8_t *>(lds);  // [64][KPL]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the wave index is the same in all 64 lanes: as a scalar it keeps the pixel-group arithmetic below
+  // (group -> image, output row, image row addresses) on the scalar unit
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 31, g = lane >> 5;
   uint32_t *patch = reinterpret_cast<uint32_t *>(lds + 64 * KPL) + wave * (R * PWD);
   const int co0 = blockIdx.y * 64;
