@@ -58,7 +58,7 @@ _CONV_NAMES = ["apconv_w1a2", "apconv_w1a3", "apconv_w1a4", "apconv_w2a2", "apco
                "apconv_w1a8", "apconv_w2a8", "APConv_w2a8_pack", "APConv_w2a8_pack_pool",
                "APConv_w1a2_pack", "APConv_w1a3_pack", "APConv_w1a4_pack", "APConv_w2a2_pack",
                "APConv_w1a2_pack_pool", "APConv_w2a2_pack_pool"]
-DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_conv_i8_bn",
+DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_pack_bits", "apnn_pack_bits_fc_hidden", "apnn_conv_i8_bn",
                                                 "apnn_pool_pack", "apnn_unpack_sum", "apnn_fc_i8",
                                                 "apnn_conv_i8_bn_pack", "apnn_pool_planes", "apnn_quantize_pack", "apnn_fold_bn", "apnn_conv_pair",
                                                 "apnn_gemm_plan", "apnn_conv_plan", "apnn_quantize_pack_u8", "apnn_binarize_pack",
@@ -120,6 +120,8 @@ def lib():
         L.apnn_conv_pair.restype = _ci
         L.apnn_pack_bits.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]
         L.apnn_pack_bits.restype = _ci
+        L.apnn_pack_bits_fc_hidden.argtypes = [_vp, _vp, _ci, _ci, _ci, _ci, _vp]
+        L.apnn_pack_bits_fc_hidden.restype = _ci
         L.apnn_conv_i8_bn.argtypes = [_vp] * 5 + [_ci] * 11 + [_vp]
         L.apnn_conv_i8_bn.restype = _ci
         L.apnn_conv_i8_bn_pack.argtypes = [_vp] * 4 + [_ci] * 11 + [_vp]

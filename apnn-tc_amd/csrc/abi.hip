@@ -770,6 +770,13 @@ int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, in
   return (int)apnn::launch_pack_bits(values, planes, rows, C, cpad, bits, static_cast<hipStream_t>(s));
 }
 
+int apnn_pack_bits_fc_hidden(const uint32_t *values, uint32_t *plane, int rows, int C, int cpad, int bits,
+                             apnn_stream_t s) {
+  if (values == nullptr || plane == nullptr) return APNN_ENULL;
+  if (rows <= 0 || C <= 0 || cpad < C || (cpad % 32) != 0 || bits < 1 || bits > 32) return APNN_EINVAL;
+  return (int)apnn::launch_pack_top_plane(values, plane, rows, C, cpad, bits, static_cast<hipStream_t>(s));
+}
+
 int apnn_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
                        float max_v, apnn_stream_t s) {
   if (values == nullptr || planes == nullptr) return APNN_ENULL;

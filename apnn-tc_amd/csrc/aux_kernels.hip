@@ -7,9 +7,10 @@ namespace apnn {
 
 // Bit-plane packer with the layout of Bit_compression (APNN-TC-nn/src/kernel.cuh:46-77):
 // one wave handles 64 consecutive channels of one row, a ballot per bit yields two MSB-first words.
+// Bits first_bit .. bits-1 of every value are written, bit b as plane b - first_bit.
 __global__ __launch_bounds__(256) void pack_bits_kernel(const uint32_t *__restrict__ values,
                                                         uint32_t *__restrict__ planes, int rows, int C,
-                                                        int cpad, int bits) {
+                                                        int cpad, int bits, int first_bit) {
   const int lane = threadIdx.x & 63;
   const int wave_in_block = threadIdx.x >> 6;
   const int cw = cpad >> 5;              // words per row
@@ -20,11 +21,11 @@ __global__ __launch_bounds__(256) void pack_bits_kernel(const uint32_t *__restri
     const int row = (int)(g / groups);
     const int c = (int)(g % groups) * 64 + lane;
     const uint32_t v = (c < C) ? values[(long long)row * C + c] : 0u;
-    for (int b = 0; b < bits; ++b) {
+    for (int b = first_bit; b < bits; ++b) {
       const unsigned long long mask = __ballot((v >> b) & 1u);
       const uint32_t word = (lane < 32) ? __brev((uint32_t)mask) : __brev((uint32_t)(mask >> 32));
       const int wi = c >> 5;
-      if ((lane & 31) == 0 && wi < cw) planes[b * plane_stride + (long long)row * cw + wi] = word;
+      if ((lane & 31) == 0 && wi < cw) planes[(b - first_bit) * plane_stride + (long long)row * cw + wi] = word;
     }
   }
 }
@@ -174,7 +175,14 @@ hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, 
   long long blocks = (total + 3) / 4;
   if (blocks > 65536) blocks = 65536;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(pack_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, s, values, planes, rows, C, cpad, bits);
+  hipLaunchKernelGGL(pack_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, s, values, planes, rows, C, cpad, bits, 0);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_top_plane(const uint32_t *values, uint32_t *plane, int rows, int C, int cpad, int bits,
+                                 hipStream_t s) {
+  hipLaunchKernelGGL(pack_bits_kernel, dim3(pack_blocks(rows, cpad)), dim3(256), 0, s, values, plane, rows, C, cpad, bits,
+                     bits - 1);
   return hipGetLastError();
 }
 

@@ -119,6 +119,8 @@ constexpr int kPatchTileCols[kPatchTileCount] = {128, 64, 128, 64, 64};
 // aux_kernels.hip
 hipError_t launch_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits,
                             hipStream_t s);
+hipError_t launch_pack_top_plane(const uint32_t *values, uint32_t *plane, int rows, int C, int cpad, int bits,
+                                 hipStream_t s);
 
 hipError_t launch_quantize_pack(const float *values, uint32_t *planes, int rows, int C, int cpad, int bits, float min_v,
                                 float max_v, hipStream_t s);

@@ -210,6 +210,14 @@ int apnn_conv_plan(const apnn_conv_desc *d, apnn_plan *plan);
  * pad channels zero.  cpad % 32 == 0, cpad >= C. */
 int apnn_pack_bits(const uint32_t *values, uint32_t *planes, int rows, int C, int cpad, int bits, apnn_stream_t s);
 
+/* Bit_compression_fc_hidden (APNN-TC-nn/src/kernel.cuh:78-126, used by weight_quantization_fc_hidden, :272):
+ * the same packer, except that the reference stores every bit-plane at the same words (the plane offset is
+ * commented out, kernel.cuh:118-123), so what its buffer holds afterwards is the plane written last, bit
+ * bits-1 of every value.  values:[rows][C] uint32 codes -> plane:[rows][cpad/32], channel c at bit 31-c%32,
+ * pad channels zero; with bits == 1 identical to apnn_pack_bits. */
+int apnn_pack_bits_fc_hidden(const uint32_t *values, uint32_t *plane, int rows, int C, int cpad, int bits,
+                             apnn_stream_t s);
+
 /* ---- layers on either side of the low-bit path ------------------------------------------------ */
 
 /* Two convolutions of the same input onto the same output grid in one launch: the entry of a residual

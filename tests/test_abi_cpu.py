@@ -43,6 +43,8 @@ def test_named_entry_points_reject_bad_arguments():
     assert L.APConv_w1a2_pack_pool(good, good, good, 15, 16, 128, 128, None) == A.EINVAL  # odd height
     assert L.apnn_pack_bits(None, good, 4, 64, 128, 2, None) == A.ENULL
     assert L.apnn_pack_bits(good, good, 4, 200, 128, 2, None) == A.EINVAL
+    assert L.apnn_pack_bits_fc_hidden(None, good, 4, 64, 128, 2, None) == A.ENULL
+    assert L.apnn_pack_bits_fc_hidden(good, good, 4, 200, 128, 2, None) == A.EINVAL
 
 
 def test_descriptor_entry_points_reject_bad_arguments():

@@ -319,6 +319,19 @@ def test_pack_bits(G):
         assert np.array_equal(got, O.pack_bits(v, rows, C, cpad, bits))
 
 
+def test_pack_bits_fc_hidden(G):
+    # the reference's loop stores all planes at the same words: the last one written (bit bits-1) stays
+    rng = np.random.default_rng(701)
+    for rows, C, cpad, bits in [(5, 3, 128, 2), (33, 70, 128, 3), (64, 192, 256, 2), (2, 100, 128, 1)]:
+        v = rng.integers(0, 2 ** bits, size=(rows, C)).astype(np.uint32)
+        dv = G.to_dev(v)
+        out = G.dev_empty_i32(rows * cpad // 32, fill=-7)
+        G.A.check(G.A.lib().apnn_pack_bits_fc_hidden(G.ptr(dv), G.ptr(out), rows, C, cpad, bits, None), "pack_fc_hidden")
+        got = G.to_host(out, np.uint32).reshape(1, rows, cpad // 32)
+        assert np.array_equal(got, O.pack_bits(v >> (bits - 1), rows, C, cpad, 1))
+        assert np.array_equal(got[0], O.pack_bits(v, rows, C, cpad, bits)[bits - 1])
+
+
 # ---- full-size shapes: size-independent properties + sampled rows ------------------------------
 
 @pytest.mark.parametrize("path", PATHS)
