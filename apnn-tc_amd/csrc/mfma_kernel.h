@@ -751,6 +751,21 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
 }
 
 
+// k-words (32 elements each) per staged chunk.  The convolution kernels whose waves tile the output
+// (64x64 and 128x64 per work-group with 128-bit loads, i.e. at least 128 stored channels; larger tiles
+// and the short reductions of narrow layers measure no gain) stage 16; so do the 256x128 GEMM tiles while
+// two work-groups' buffers still fit a compute unit (three planes in all: w1a2, -4 % at 4096^3 / 8192^3;
+// with four planes the larger buffers leave one work-group per unit and cost 28 %); the split-K tiles, used
+// for few outputs over a long K where every chunk iteration is a latency chain, stage 32: their per-chunk
+// work (im2col addressing, LDS staging, barrier) is a large share of a short K loop, and k-steps past the
+// end of K are skipped, so a longer chunk wastes nothing.
+constexpr int mfma_chunk_words(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
+  if (WA * WB == 1) return 32;
+  if (conv && FA * FB <= 2 && vw == 4) return 16;
+  if (!conv && FA * FB >= 8 && (PA * WA * FA + PB * WB * FB) * 32 <= 512) return 16;
+  return 8;
+}
+
 // longest reduction (32-bit words) the one- and two-block convolution tiles load without staging
 constexpr int kDirectMaxKW = 40;
 
@@ -783,12 +798,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   using FragT = typename std::conditional<F4, v8i, v4i>::type;
   constexpr int NT = 256;
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  // k-words (32 elements each) per staged chunk.  The convolution kernels whose waves tile the output
-  // (64x64 and 128x64 per work-group with 128-bit loads, i.e. at least 128 stored channels; larger tiles
-  // and the short reductions of narrow layers measure no gain) stage 16; the split-K tiles, used for
-  // few outputs over a long K where every chunk iteration is a latency chain, stage 32: their per-chunk work (im2col addressing, LDS staging, barrier) is a large share of a
-  // short K loop, and k-steps past the end of K are skipped, so a longer chunk wastes nothing.
-  constexpr int KC = KS > 1 ? 32 : (CONV && FA * FB <= 2 && VW == 4) ? 16 : 8;
+  constexpr int KC = mfma_chunk_words(PA, PB, FA, FB, WA, WB, CONV, VW);
   constexpr int LD = KC + 1;         // odd row pitch: 32 rows hit 32 different banks
   constexpr int KQ = KC / VW;
   constexpr int UA = TA * KQ, UB = TB * KQ;
@@ -1194,7 +1204,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
 }
 
 constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
-  const size_t ld = WA * WB == 1 ? 33 : (conv && FA * FB <= 2 && vw == 4) ? 17 : 9;  // KC + 1, see the kernel
+  const size_t ld = mfma_chunk_words(PA, PB, FA, FB, WA, WB, conv, vw) + 1;
   // FP4 split-K tiles with 128-bit loads stage nothing (operands go from global memory to registers)
   const size_t stage = core == CORE_F4 && WA * WB == 1 && vw == 4
                            ? 0
