@@ -278,7 +278,7 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3, bool int32_out = false) {
   const bool wide = planes > 5;
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -317,7 +317,10 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
     // compute unit (7x7x512 maps at batch 64, 16x16x512..1024 at batch 16): one activation expansion feeds
     // four blocks, 11-16 % faster than 32x64 / 128x64 there; with 256 channels or fewer tiles it loses
     if (vw == 4 && KW >= 64 && rowsB >= 512 && 2 * ntiles(8) >= 3 * cus && nb32 <= 4096) return 8;
-    if (KW >= 32 && nb32 <= 256) return 4;   // at most one work-group per compute unit
+    // quantized output: up to two 32x32 work-groups per compute unit (measured 6-11 % ahead of 32x64 at 392
+    // and 512 blocks); int32 output, whose split-K store goes through LDS: at most one (32x64 is 10 % ahead
+    // at 512 blocks)
+    if (KW >= 32 && nb32 <= (int32_out ? 256 : 512)) return 4;
     if (KW >= 32 && nb32 <= 640) return 5;
     if (KW >= 64 && nb32 <= 3200) return 5;
   }
@@ -345,7 +348,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
 
 int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB, p.epi == APNN_EPI_INT32);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
