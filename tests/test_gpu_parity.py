@@ -80,16 +80,17 @@ def test_gemm_sweep_m64(G, wb, xb, nk, path):
     assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, nthreads=8))
 
 
+@pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("path,tile", GEMM_TILES)
 @pytest.mark.parametrize("wb,xb", COMBOS)
-def test_gemm_every_tile_ragged(G, wb, xb, tile, path):
-    """Row / column counts that are not multiples of any tile, every tile shape pinned."""
+def test_gemm_every_tile_ragged(G, wb, xb, tile, path, sym):
+    """Row / column counts that are not multiples of any tile, every tile shape pinned, both weight modes."""
     rng = np.random.default_rng(50 + tile + 10 * wb + xb)
     M, N, K = (70, 97, 384) if path == 1 else (300, 289, 640)
     W = O.random_planes(rng, wb, M, K // 32)
     X = O.random_planes(rng, xb, N, K // 32)
-    got = G.run_gemm(W, X, M, N, K, wb, xb, path=path, tile=tile).reshape(M, N)
-    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb))
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=sym, path=path, tile=tile).reshape(M, N)
+    assert np.array_equal(got, O.gemm(W, X, M, N, K, wb, xb, sym_w=sym))
 
 
 @pytest.mark.parametrize("path", PATHS)
