@@ -1016,9 +1016,73 @@ hipError_t launch_unpack_sum(const uint32_t *planes, int8_t *out, long long rows
   return hipGetLastError();
 }
 
+// Larger batches: one wave per 8 output features x 8 batch rows (every operand dword is used eight times, so
+// the waves re-read half as many bytes from L2 as with 4 x 4).  The 64 per-lane partial sums are reduced
+// by a transposing butterfly: at step s a lane keeps the accumulator whose index has bit s equal to its own
+// lane bit s and hands the other one to its partner lane, so the number of live accumulators halves at every
+// step (63 exchanges in all instead of 6 x 64) and lane l ends up with the complete sum of accumulator l.
+// Requires K % 4 == 0 and 4-byte aligned rows.
+__global__ __launch_bounds__(256) void fc_i8_tile_kernel(const int8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+                                                         const float *__restrict__ scale, const float *__restrict__ bias,
+                                                         float *__restrict__ out, int32_t *__restrict__ acc_out, int Bn,
+                                                         int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int bgroups = (Bn + 7) >> 3, ngroups = (N + 7) >> 3;
+  const long long wid = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wid >= (long long)ngroups * bgroups) return;
+  const int n0 = (int)(wid % ngroups) * 8;
+  const int b0 = (int)(wid / ngroups) * 8;
+  int acc[64];
+#pragma unroll
+  for (int a = 0; a < 64; ++a) acc[a] = 0;
+  const int *wrow[8], *xrow[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    wrow[i] = reinterpret_cast<const int *>(Wt + (long long)min(n0 + i, N - 1) * K);
+    xrow[i] = reinterpret_cast<const int *>(X + (long long)min(b0 + i, Bn - 1) * K);
+  }
+#pragma unroll 2
+  for (int k4 = lane; k4 < (K >> 2); k4 += 64) {
+    int wv[8], xv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      wv[i] = wrow[i][k4];
+      xv[i] = xrow[i][k4];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i * 8 + j] = __builtin_amdgcn_sdot4(xv[j], wv[i], acc[i * 8 + j], false);
+  }
+  static_for_n<0, 6>([&](auto sc) {
+    constexpr int st = decltype(sc)::value;
+    constexpr int n = 64 >> st;  // live accumulators before this step
+    const bool hi = (lane >> st) & 1;
+#pragma unroll
+    for (int t = 0; t < n / 2; ++t) {
+      const int keep = hi ? acc[2 * t + 1] : acc[2 * t];
+      const int send = hi ? acc[2 * t] : acc[2 * t + 1];
+      acc[t] = keep + __shfl_xor(send, 1 << st, 64);
+    }
+  });
+  // lane l = 8 * feature + batch row (rows / features past the end were clamped duplicates: dropped here)
+  const int i = lane >> 3, j = lane & 7;
+  if (n0 + i < N && b0 + j < Bn) {
+    const long long o = (long long)(b0 + j) * N + n0 + i;
+    if (acc_out != nullptr) acc_out[o] = acc[0];
+    out[o] = (float)acc[0] * scale[n0 + i] + bias[n0 + i];
+  }
+}
+
 hipError_t launch_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
                         int32_t *acc_out, int Bn, int N, int K, hipStream_t s) {
   const int vec_ok = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Wt)) & 3u) == 0;
+  if (vec_ok && Bn >= 32 && (long long)((N + 7) / 8) * ((Bn + 7) / 8) >= 512) {
+    const long long waves = (long long)((N + 7) / 8) * ((Bn + 7) / 8);
+    hipLaunchKernelGGL(fc_i8_tile_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out,
+                       acc_out, Bn, N, K);
+    return hipGetLastError();
+  }
   if ((long long)N * ((Bn + 3) / 4) >= 8192) {  // plenty of waves: four features per wave cut the re-reads of X
     const long long waves = (long long)((N + 3) / 4) * ((Bn + 3) / 4);
     hipLaunchKernelGGL(fc_i8_kernel<4>, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, X, Wt, scale, bias, out,

@@ -450,6 +450,27 @@ def test_unpack_sum_and_fc_i8(G):
     assert np.allclose(d_out.cpu().numpy().reshape(B, N), expect, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("Bn,N,K", [(64, 1000, 512), (64, 1000, 4096), (37, 1003, 516), (32, 130, 64), (8, 1000, 512),
+                                    (40, 50, 128), (33, 999, 510)])
+def test_fc_i8_batches(G, Bn, N, K):
+    """int8 classifier at the batch sizes of the networks: the 8 x 8-tile kernel (batch >= 32, whole dwords),
+    ragged feature / batch / K counts, and the shapes that stay on the smaller kernels."""
+    rng = np.random.default_rng(960 + Bn + N + K)
+    X = rng.integers(-128, 128, size=(Bn, K)).astype(np.int8)
+    Wt = rng.integers(-128, 128, size=(N, K)).astype(np.int8)
+    scale = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    d_out = torch.empty(Bn * N, dtype=torch.float32, device="cuda")
+    d_acc = G.dev_empty_i32(Bn * N, fill=-7)
+    dX, dW, dS, dB = G.to_dev(X), G.to_dev(Wt), torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
+    G.A.check(G.A.lib().apnn_fc_i8(G.ptr(dX), G.ptr(dW), G.ptr(dS), G.ptr(dB), G.ptr(d_out), G.ptr(d_acc), Bn, N, K, None), "fc")
+    acc = X.astype(np.int64) @ Wt.astype(np.int64).T
+    assert np.array_equal(G.to_host(d_acc).reshape(Bn, N), acc)
+    torch.cuda.synchronize()
+    expect = acc.astype(np.float32) * scale[None, :] + bias[None, :]
+    assert np.allclose(d_out.cpu().numpy().reshape(Bn, N), expect, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("B,HW,C,cpad,bits,shift", [(3, 150, 96, 96, 3, 2), (2, 64, 40, 64, 1, 0), (5, 9, 64, 64, 4, 0),
                                                     (2, 7, 33, 64, 2, 0)])
 def test_unpack_sum_group_sizes(G, B, HW, C, cpad, bits, shift):
