@@ -132,3 +132,69 @@ def test_gemm_random_shapes(G, block):
         ran += 1
         assert got.shape == expect.shape and np.array_equal(got, expect), case
     assert ran >= 30
+
+
+def _np_maxpool_codes(codes, win, stride, pad):
+    B, H, W, C = codes.shape
+    Ho, Wo = (H + 2 * pad - win) // stride + 1, (W + 2 * pad - win) // stride + 1
+    padded = np.full((B, H + 2 * pad, W + 2 * pad, C), -1, codes.dtype)
+    padded[:, pad:pad + H, pad:pad + W] = codes
+    out = np.full((B, Ho, Wo, C), -1, codes.dtype)
+    for r in range(win):
+        for s in range(win):
+            out = np.maximum(out, padded[:, r:r + stride * Ho:stride, s:s + stride * Wo:stride])
+    return out
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_first_layer_and_plane_pool_random_shapes(G, block):
+    """int8 first layer (thresholds and bit-plane packing fused) on drawn image sizes, channel counts,
+    filters, strides and paddings, then the max-pool on its bit-planes with a drawn window."""
+    L = G.A.lib()
+    ran = 0
+    for i in range(40):
+        rng = np.random.default_rng(910000 + 1000 * block + i)
+        B = int(rng.integers(1, 5))
+        H, Wd = int(rng.integers(8, 80)), int(rng.integers(8, 140))
+        if rng.random() < 0.5:
+            Wd = (Wd + 3) // 4 * 4            # rows of a multiple of four bytes take the byte-row kernel
+        C = int(rng.integers(1, 5))
+        cout = int(rng.choice([32, 64, 64, 96, 128]))
+        R = int(rng.choice([3, 5, 7, 7, 11]))
+        stride = int(rng.integers(1, 5))
+        pad = int(rng.integers(0, R // 2 + 1))
+        bits = int(rng.integers(1, 5))
+        zero_point = int(rng.choice([0, 128]))
+        if H + 2 * pad < R or Wd + 2 * pad < R:
+            continue
+        case = dict(block=block, i=i, B=B, H=H, W=Wd, C=C, cout=cout, R=R, stride=stride, pad=pad, bits=bits, zp=zero_point)
+        if zero_point:
+            Xraw = rng.integers(0, 256, size=(B, H, Wd, C)).astype(np.uint8)
+            Xs = (Xraw.astype(np.int16) - zero_point).astype(np.int8)
+        else:
+            Xs = rng.integers(-128, 128, size=(B, H, Wd, C)).astype(np.int8)
+            Xraw = Xs
+        Wt = rng.integers(-128, 128, size=(cout, R, R, C)).astype(np.int8)
+        acc = O.conv_i8(Wt, Xs, stride, pad)
+        Ho, Wo = acc.shape[1], acc.shape[2]
+        rows = B * Ho * Wo
+        span = max(1, int(np.abs(acc).max()))
+        thr = np.sort(rng.integers(-span, span + 1, size=(cout, 2 ** bits - 1)), axis=1).astype(np.int32)
+        codes = O.bn_quantize(acc.reshape(-1, cout), None, thr, None, bits).reshape(acc.shape)
+        dX, dW, dT = torch.from_numpy(Xraw).cuda(), G.to_dev(Wt), G.to_dev(thr)
+        d_planes = G.dev_empty_i32(bits * rows * cout // 32, fill=-7)
+        G.A.check(L.apnn_conv_i8_bn_pack(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_planes), B, H, Wd, C, cout, R, R,
+                                         stride, pad, bits, zero_point, None), "conv_i8_bn_pack %r" % (case,))
+        ran += 1
+        expect = O.pack_bits(codes.reshape(rows, cout).astype(np.uint32), rows, cout, cout, bits)
+        assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect), case
+        win, st, pd = [(3, 2, 1), (2, 2, 0), (3, 1, 1), (2, 1, 0), (3, 3, 0)][rng.integers(0, 5)]
+        if Ho + 2 * pd < win or Wo + 2 * pd < win:
+            continue
+        pooled = _np_maxpool_codes(codes, win, st, pd)
+        prow = pooled.shape[0] * pooled.shape[1] * pooled.shape[2]
+        d_out = G.dev_empty_i32(bits * prow * cout // 32, fill=-7)
+        G.A.check(L.apnn_pool_planes(G.ptr(d_planes), G.ptr(d_out), B, Ho, Wo, cout, bits, win, st, pd, None), "pool_planes")
+        pexp = O.pack_bits(pooled.reshape(prow, cout).astype(np.uint32), prow, cout, cout, bits)
+        assert np.array_equal(G.to_host(d_out, np.uint32).reshape(pexp.shape), pexp), (case, win, st, pd)
+    assert ran >= 20
