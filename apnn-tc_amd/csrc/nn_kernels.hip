@@ -318,10 +318,21 @@ __device__ __forceinline__ void static_for_n(F &&f) {
   }
 }
 
-// old with lane LANE replaced by the wave-uniform value val
-template <int LANE>
-__device__ __forceinline__ int write_lane_n(int val, int old) {
-  asm("v_writelane_b32 %0, %1, %2" : "+v"(old) : "s"(val), "n"(LANE));
+// old with lanes L0, L0 + 4 replaced by the halves of m0 and lanes L0 + 32, L0 + 36 by the halves of m1
+// (wave-uniform compare masks).  A vector instruction that takes a scalar register written by the vector
+// instruction just before it needs two wait states, which the compiler inserts only for instructions it
+// can see -- not for this opaque assembly, hence the leading s_nop.
+template <int L0>
+__device__ __forceinline__ int write_mask_lanes(unsigned long long m0, unsigned long long m1, int old) {
+  static_assert(L0 >= 0 && L0 + 36 < 64, "lane index");
+  asm("s_nop 1\n\t"
+      "v_writelane_b32 %0, %1, %5\n\t"
+      "v_writelane_b32 %0, %2, %6\n\t"
+      "v_writelane_b32 %0, %3, %7\n\t"
+      "v_writelane_b32 %0, %4, %8"
+      : "+v"(old)
+      : "s"((int)(uint32_t)m0), "s"((int)(uint32_t)(m0 >> 32)), "s"((int)(uint32_t)m1), "s"((int)(uint32_t)(m1 >> 32)),
+        "n"(L0), "n"(L0 + 4), "n"(L0 + 32), "n"(L0 + 36));
   return old;
 }
 
@@ -336,7 +347,9 @@ __device__ __forceinline__ int write_lane_n(int val, int old) {
 // aligned dword reads and four v_alignbyte.  With NKS > 0 the wave keeps its 64 x (NKS*32) weight
 // block in registers for the whole (persistent) kernel; with NKS == 0 weights are read from LDS.
 // The epilogue is the compare-is-ballot scheme of the matrix-core kernels: per accumulator register
-// two compares and a select give both bit-plane masks of two output pixels.
+// two compares and a select give both bit-plane masks of two output pixels.  Lane li of a column block
+// works on output channel 31 - li (its filter row and thresholds are read in that order), so a compare
+// mask already is the packed word (channel c at bit 31 - c%32) and needs no bit reversal.
 // Requires C <= 4, (W*C) % 4 == 0, X 4-byte aligned, bits <= 2, COUT % 32 == 0.
 // NWAV waves per work-group share one filter block in LDS (each wave has its own patch and walks its
 // own pixel groups): eight waves where the filter block is large, so that its LDS cost per wave halves
@@ -419,7 +432,7 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
     for (int ks = 0; ks < NW; ++ks) {
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
-        wreg[nb][ks] = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KPL + ks * 32 + g * 16);
+        wreg[nb][ks] = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + 31 - li) * KPL + ks * 32 + g * 16);
       const int hh = 2 * ks + g;
       const int r = min(hh / HPR, R - 1);
       koff[ks] = r * PWD * 4 + (hh % HPR) * 16;
@@ -430,7 +443,7 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
   int t0[2], t1[2], t2[2];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const int co = co0 + nb * 32 + li;
+    const int co = co0 + nb * 32 + 31 - li;
     t0[nb] = t1[nb] = t2[nb] = 0x7fffffff;
     if (co < COUT) {
       t0[nb] = thr[co * nt];
@@ -459,7 +472,11 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
     const int r = (int)quot((uint32_t)idx, (uint32_t)NDW, magic_ndw);
     rd[j] = idx < npatch ? ((r << 16) | (idx - r * NDW)) : -1;
   }
+  // Loads are unconditional (addresses clamped into the image) and leave the registers untouched until
+  // publish(): a load whose value is used inside a branch on its predicate makes the compiler wait
+  // for it there, one memory round trip per slot.  raw_ok bit j: slot j lies inside the image.
   uint32_t raw[NSLOT];
+  uint32_t raw_ok = 0;
   auto request = [&](uint32_t grp, int base) {
     const uint32_t trow = quot(grp, (uint32_t)gpr, magic_gpr);
     const int gx = (int)(grp - trow * (uint32_t)gpr);
@@ -467,6 +484,7 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
     const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
     const int sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
     const uint8_t *img = X + (long long)b * H * rowbytes;
+    uint32_t okbits = 0;
 #pragma unroll
     for (int j = 0; j < NSLOT; ++j) {
       int r, d;
@@ -484,18 +502,22 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
       const int iy = oy * stride - pad + r;
       const int sb = sbase + 4 * d;
       ok = ok && iy >= 0 && iy < H && sb >= 0 && sb < rowbytes;
-      raw[j] = ok ? (*reinterpret_cast<const uint32_t *>(img + (long long)iy * rowbytes + sb) ^ xor_mask) : 0u;
+      const int iyc = min(max(iy, 0), H - 1), sbc = min(max(sb, 0), rowbytes - 4);
+      raw[j] = *reinterpret_cast<const uint32_t *>(img + (long long)iyc * rowbytes + sbc);
+      okbits |= ok ? (1u << j) : 0u;
     }
+    raw_ok = okbits;
   };
   auto publish = [&](int base) {
 #pragma unroll
     for (int j = 0; j < NSLOT; ++j) {
+      const uint32_t val = (raw_ok >> j) & 1u ? raw[j] ^ xor_mask : 0u;
       if (base == 0) {
-        if (rd[j] >= 0) patch[(rd[j] >> 16) * PWD + (rd[j] & 0xffff)] = raw[j];
+        if (rd[j] >= 0) patch[(rd[j] >> 16) * PWD + (rd[j] & 0xffff)] = val;
       } else {
         const int idx = base + j * 64 + lane;
         const int r = idx / NDW;
-        if (idx < npatch) patch[r * PWD + (idx - r * NDW)] = raw[j];
+        if (idx < npatch) patch[r * PWD + (idx - r * NDW)] = val;
       }
     }
   };
@@ -557,7 +579,7 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
         const v4i_t af = operand(min(r, R - 1) * PWD * 4 + h * 16);
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-          const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + li) * KPL + ks * 32 + g * 16);
+          const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + 31 - li) * KPL + ks * 32 + g * 16);
           acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[nb], 0, 0, 0);
         }
         h += 2;
@@ -574,18 +596,13 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
     for (int nb = 0; nb < 2; ++nb) {
       static_for_n<0, 16>([&](auto rc) {
         constexpr int r = decltype(rc)::value;
-        constexpr int rlo = 8 * (r >> 2) + (r & 3), rhi = rlo + 4;
+        constexpr int rlo = 8 * (r >> 2) + (r & 3);  // lane half 0's pixel; lane half 1's is rlo + 4
         const int v = acc[nb][r];
         const bool hi1 = v >= t1[nb];
         const unsigned long long m1 = __ballot(hi1);
         const int tsel = hi1 ? t2[nb] : t0[nb];
         const unsigned long long m0 = __ballot(v >= tsel);
-        int reg = park[nb];
-        reg = write_lane_n<rlo>((int)__brev((uint32_t)m0), reg);
-        reg = write_lane_n<rhi>((int)__brev((uint32_t)(m0 >> 32)), reg);
-        reg = write_lane_n<rlo + 32>((int)__brev((uint32_t)m1), reg);
-        reg = write_lane_n<rhi + 32>((int)__brev((uint32_t)(m1 >> 32)), reg);
-        park[nb] = reg;
+        park[nb] = write_mask_lanes<rlo>(m0, m1, park[nb]);
       });
     }
     const int ox = ox0 + li, plane = g;
