@@ -465,67 +465,75 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
   // group is computed (patches of up to 64 * NSLOT dwords: NSLOT = 8 covers a 7x7 stride-2 filter on
   // three channels, 18 an 11x11 stride-4 one; larger patches are staged in place, chunk by chunk).
   const bool prefetch = npatch <= 64 * NSLOT;
+  // rd[j]: row segment r in the upper half-word, byte offset 4*d in the lower one; r = NO_ROW marks a
+  // slot past the end of the patch (it then fails the row test of every group)
+  constexpr int NO_ROW = 0x7fff;
+  auto slot_code = [&](int idx) {
+    const int r = (int)quot((uint32_t)idx, (uint32_t)NDW, magic_ndw);
+    return idx < npatch ? ((r << 16) | (4 * (idx - r * NDW))) : (NO_ROW << 16);
+  };
   int rd[NSLOT];
 #pragma unroll
-  for (int j = 0; j < NSLOT; ++j) {
-    const int idx = j * 64 + lane;
-    const int r = (int)quot((uint32_t)idx, (uint32_t)NDW, magic_ndw);
-    rd[j] = idx < npatch ? ((r << 16) | (idx - r * NDW)) : -1;
-  }
+  for (int j = 0; j < NSLOT; ++j) rd[j] = slot_code(j * 64 + lane);
   // Loads are unconditional (addresses clamped into the image) and leave the registers untouched until
   // publish(): a load whose value is used inside a branch on its predicate makes the compiler wait
-  // for it there, one memory round trip per slot.  raw_ok bit j: slot j lies inside the image.
+  // for it there, one memory round trip per slot.  raw_ok[j]: slot j lies inside the image.  The address
+  // is the image's base (uniform) plus a 32-bit byte offset, seven vector operations per slot: row and
+  // byte position, two range tests, two clamps, one multiply-add (the launcher checks H * W * C < 2^31,
+  // W * C < 2^24 and H + pad < NO_ROW).
   uint32_t raw[NSLOT];
-  uint32_t raw_ok = 0;
-  auto request = [&](uint32_t grp, int base) {
+  bool raw_ok[NSLOT];
+  // one patch dword of pixel group grp: image dword and whether it lies inside the image
+  auto load_slot = [&](const uint8_t *img, int ybase, int sbase, int code, uint32_t &word, bool &inside) {
+    const int iy = ybase + (code >> 16);
+    const int sb = sbase + (code & 0xffff);
+    inside = (uint32_t)iy < (uint32_t)H && (uint32_t)sb < (uint32_t)rowbytes;
+    const int iyc = min(max(iy, 0), H - 1), sbc = min(max(sb, 0), rowbytes - 4);
+    const uint32_t off = __umul24((uint32_t)iyc, (uint32_t)rowbytes) + (uint32_t)sbc;
+    word = *reinterpret_cast<const uint32_t *>(img + off);
+  };
+  auto group_origin = [&](uint32_t grp, const uint8_t *&img, int &ybase, int &sbase) {
     const uint32_t trow = quot(grp, (uint32_t)gpr, magic_gpr);
     const int gx = (int)(grp - trow * (uint32_t)gpr);
     const int b = (int)quot(trow, (uint32_t)Ho, magic_ho);
     const int oy = (int)(trow - (uint32_t)b * (uint32_t)Ho);
-    const int sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
-    const uint8_t *img = X + (long long)b * H * rowbytes;
-    uint32_t okbits = 0;
-#pragma unroll
-    for (int j = 0; j < NSLOT; ++j) {
-      int r, d;
-      bool ok;
-      if (base == 0) {
-        r = rd[j] >> 16;
-        d = rd[j] & 0xffff;
-        ok = rd[j] >= 0;
-      } else {
-        const int idx = base + j * 64 + lane;
-        r = idx / NDW;
-        d = idx - r * NDW;
-        ok = idx < npatch;
-      }
-      const int iy = oy * stride - pad + r;
-      const int sb = sbase + 4 * d;
-      ok = ok && iy >= 0 && iy < H && sb >= 0 && sb < rowbytes;
-      const int iyc = min(max(iy, 0), H - 1), sbc = min(max(sb, 0), rowbytes - 4);
-      raw[j] = *reinterpret_cast<const uint32_t *>(img + (long long)iyc * rowbytes + sbc);
-      okbits |= ok ? (1u << j) : 0u;
-    }
-    raw_ok = okbits;
+    sbase = ((gx * 32 * stride - pad) * C) & ~3;  // two's complement: rounds towards minus infinity
+    ybase = oy * stride - pad;
+    img = X + (long long)b * H * rowbytes;
   };
-  auto publish = [&](int base) {
+  auto request = [&](uint32_t grp) {
+    const uint8_t *img;
+    int ybase, sbase;
+    group_origin(grp, img, ybase, sbase);
+#pragma unroll
+    for (int j = 0; j < NSLOT; ++j) load_slot(img, ybase, sbase, rd[j], raw[j], raw_ok[j]);
+  };
+  auto publish = [&]() {
 #pragma unroll
     for (int j = 0; j < NSLOT; ++j) {
-      const uint32_t val = (raw_ok >> j) & 1u ? raw[j] ^ xor_mask : 0u;
-      if (base == 0) {
-        if (rd[j] >= 0) patch[(rd[j] >> 16) * PWD + (rd[j] & 0xffff)] = val;
-      } else {
-        const int idx = base + j * 64 + lane;
-        const int r = idx / NDW;
-        if (idx < npatch) patch[r * PWD + (idx - r * NDW)] = val;
-      }
+      const uint32_t val = raw_ok[j] ? raw[j] ^ xor_mask : 0u;
+      if (rd[j] < (NO_ROW << 16)) patch[(rd[j] >> 16) * PWD + ((rd[j] & 0xffff) >> 2)] = val;
+    }
+  };
+  // patches larger than the slots: staged in place, one dword per lane and round trip
+  auto stage_in_place = [&](uint32_t grp) {
+    const uint8_t *img;
+    int ybase, sbase;
+    group_origin(grp, img, ybase, sbase);
+#pragma unroll 1
+    for (int idx = lane; idx < npatch; idx += 64) {
+      const int code = slot_code(idx);
+      uint32_t word;
+      bool inside;
+      load_slot(img, ybase, sbase, code, word, inside);
+      patch[(code >> 16) * PWD + ((code & 0xffff) >> 2)] = inside ? word ^ xor_mask : 0u;
     }
   };
 
   // (the launcher keeps the number of groups below 2^31: 32-bit index arithmetic)
   const uint32_t gstep = gridDim.x * (uint32_t)NWAV, ng = (uint32_t)ngroups;
   uint32_t group = blockIdx.x * (uint32_t)NWAV + (uint32_t)wave;
-  if (prefetch && group < ng) request(group, 0);
+  if (prefetch && group < ng) request(group);
   for (; group < ng; group += gstep) {
     const uint32_t trow = quot(group, (uint32_t)gpr, magic_gpr);
     const int gx = (int)(group - trow * (uint32_t)gpr);
@@ -535,13 +543,10 @@ __global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *
     const int s0 = (ox0 * stride - pad) * C;
     const int lead = s0 - (s0 & ~3);
     if (prefetch) {
-      publish(0);
-      if (group + gstep < ng) request(group + gstep, 0);
+      publish();
+      if (group + gstep < ng) request(group + gstep);
     } else {
-      for (int base = 0; base < npatch; base += 64 * NSLOT) {
-        request(group, base);
-        publish(base);
-      }
+      stage_in_place(group);
     }
 
     v16i_t acc[2];
@@ -886,8 +891,8 @@ hipError_t launch_conv_i8_bn(const int8_t *X, const int8_t *Wt, const int32_t *t
   const long long groups = (long long)B * Ho * ((Wo + 31) / 32);
   dim3 grid((unsigned)((groups + 3) / 4), (unsigned)((COUT + 63) / 64));
   if (C <= 4 && planes != nullptr && codes == nullptr && acc_out == nullptr && bits <= 2 && (COUT % 32) == 0 &&
-      groups < 0x7fffffffLL &&
-      ((W * C) % 4) == 0 && (reinterpret_cast<uintptr_t>(X) & 3u) == 0 && (zero_point == 0 || zero_point == 128) &&
+      groups < 0x7fffffffLL && (long long)H * W * C < 0x7fffffffLL && (long long)W * C < (1 << 24) &&
+      (long long)H + pad < 0x7fff && ((W * C) % 4) == 0 && (reinterpret_cast<uintptr_t>(X) & 3u) == 0 && (zero_point == 0 || zero_point == 128) &&
       thr != nullptr) {
     // image rows consumed as bytes (no repacking): see conv_i8_rows_kernel
     const int HPR = (S * C + 15) / 16;
