@@ -842,6 +842,15 @@ __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X
   for (int i = 0; i < NN; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0;
+  // the affine map of this wave's features, requested before the K loop (clamped index, no branch) so
+  // that the epilogue does not pay a memory round trip per output
+  float sc[NN], bi[NN];
+#pragma unroll
+  for (int i = 0; i < NN; ++i) {
+    const int n = min(n0 + i, N - 1);
+    sc[i] = scale[n];
+    bi[i] = bias[n];
+  }
   if (vec_ok) {
     // four independent iterations in flight: a long K would otherwise be one memory round trip per step
 #pragma unroll 4
@@ -878,7 +887,7 @@ __global__ __launch_bounds__(256) void fc_i8_kernel(const int8_t *__restrict__ X
       if (lane == 0 && b0 + j < Bn && n0 + i < N) {
         const long long o = (long long)(b0 + j) * N + n0 + i;
         if (acc_out != nullptr) acc_out[o] = acc[i][j];
-        out[o] = (float)acc[i][j] * scale[n0 + i] + bias[n0 + i];
+        out[o] = (float)acc[i][j] * sc[i] + bi[i];
       }
     }
 }
@@ -1057,6 +1066,9 @@ __global__ __launch_bounds__(256) void fc_i8_tile_kernel(const int8_t *__restric
   int acc[64];
 #pragma unroll
   for (int a = 0; a < 64; ++a) acc[a] = 0;
+  // the affine map of this lane's output feature, requested before the K loop
+  const int nf = min(n0 + (lane >> 3), N - 1);
+  const float out_scale = scale[nf], out_bias = bias[nf];
   const int *wrow[8], *xrow[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -1092,7 +1104,7 @@ __global__ __launch_bounds__(256) void fc_i8_tile_kernel(const int8_t *__restric
   if (n0 + i < N && b0 + j < Bn) {
     const long long o = (long long)(b0 + j) * N + n0 + i;
     if (acc_out != nullptr) acc_out[o] = acc[0];
-    out[o] = (float)acc[0] * scale[n0 + i] + bias[n0 + i];
+    out[o] = (float)acc[0] * out_scale + out_bias;
   }
 }
 
