@@ -353,9 +353,10 @@ __device__ __forceinline__ int write_mask_lanes(unsigned long long m0, unsigned 
 // Requires C <= 4, (W*C) % 4 == 0, X 4-byte aligned, bits <= 2, COUT % 32 == 0.
 // NWAV waves per work-group share one filter block in LDS (each wave has its own patch and walks its
 // own pixel groups): eight waves where the filter block is large, so that its LDS cost per wave halves
-// and four waves per SIMD stay resident.
+// and four waves per SIMD stay resident (two work-groups per compute unit: the register budget of that
+// variant is held to 128 by its launch bounds).
 template <int NKS, int NSLOT, int NWAV>
-__global__ __launch_bounds__(64 * NWAV) void conv_i8_rows_kernel(const uint8_t *__restrict__ X, const int8_t *__restrict__ Wt,
+__global__ __launch_bounds__(64 * NWAV, NWAV == 8 ? 4 : 1) void conv_i8_rows_kernel(const uint8_t *__restrict__ X, const int8_t *__restrict__ Wt,
                                                            const int32_t *__restrict__ thr,
                                                            uint32_t *__restrict__ planes, int B, int H, int W, int C,
                                                            int COUT, int R, int S, int stride, int pad, int Ho, int Wo,
