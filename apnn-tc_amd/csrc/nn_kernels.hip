@@ -581,19 +581,23 @@ __global__ __launch_bounds__(64 * NWAV, NWAV == 8 ? 4 : 1) void conv_i8_rows_ker
         h -= HPR;
         ++r;
       }
-      for (int ks = 0; ks < nks; ++ks) {
+      // k-step 0 is peeled: its matrix instructions take the constant zero as their addend, which saves
+      // clearing 32 accumulator registers per pixel group (this loop's trip count is a run-time value)
+      auto k_step = [&](int ks, const v16i_t &c0, const v16i_t &c1) {
         const v4i_t af = operand(min(r, R - 1) * PWD * 4 + h * 16);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-          const v4i_t bf = *reinterpret_cast<const v4i_t *>(wl + (nb * 32 + 31 - li) * KPL + ks * 32 + g * 16);
-          acc[nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[nb], 0, 0, 0);
-        }
+        const v4i_t b0 = *reinterpret_cast<const v4i_t *>(wl + (31 - li) * KPL + ks * 32 + g * 16);
+        const v4i_t b1 = *reinterpret_cast<const v4i_t *>(wl + (63 - li) * KPL + ks * 32 + g * 16);
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b0, c0, 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b1, c1, 0, 0, 0);
         h += 2;
         while (h >= HPR) {
           h -= HPR;
           ++r;
         }
-      }
+      };
+      const v16i_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      k_step(0, zero, zero);
+      for (int ks = 1; ks < nks; ++ks) k_step(ks, acc[0], acc[1]);
     }
 
     // ---- thresholds -> bit-plane words, parked at lane = pixel (+32 for plane 1) -------------------
