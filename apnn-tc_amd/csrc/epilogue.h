@@ -174,7 +174,6 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
   for (int u0 = part; u0 < nunits; u0 += nparts * UB) {
     int v[UB], grow[UB], gcol[UB];
     bool ok[UB];
-    uint32_t rw[UB][8];
     int ri[UB];
 #pragma unroll
     for (int j = 0; j < UB; ++j) {
@@ -188,10 +187,6 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
       if (ok[j] && !pooled) {
         const long long o = (long long)grow[j] * p.rowsB + gcol[j];
         if (p.resid != nullptr) ri[j] = p.resid[o];
-        if (res_global) {
-          const long long wi = (long long)grow[j] * w32 + (gcol[j] >> 5);
-          for (int b = 0; b < p.resid_bits; ++b) rw[j][b] = p.resid_planes[b * rplane + wi];
-        }
       }
     }
 #pragma unroll
@@ -207,8 +202,15 @@ __device__ __forceinline__ void pack_rows(const KParams &p, ValueFn value, int n
           if (res_global || res_local) {
             const int sh = 31 - (gcol[j] & 31);
             int rc = 0;
+            // Shortcut words that were not brought to LDS before the K loop (codes wider than two bits)
+            // are read here, one plane at a time.  They are not buffered in a per-lane array: indexed by
+            // a run-time plane count it would live in scratch memory, and held in registers it would
+            // spill at these kernels' register caps; this way most instantiations use no scratch at all.
+            const long long wi = (long long)grow[j] * w32 + (gcol[j] >> 5);
             for (int b = 0; b < p.resid_bits; ++b) {
-              const uint32_t w = res_local ? res_lds[(b * n_rows + orow) * (NCOLS / 32) + (col >> 5)] : rw[j][b];
+              uint32_t w = 0;
+              if (res_local) w = res_lds[(b * n_rows + orow) * (NCOLS / 32) + (col >> 5)];
+              if (res_global) w = p.resid_planes[b * rplane + wi];
               rc |= (int)((w >> sh) & 1u) << b;
             }
             t += rc * p.resid_scale;
