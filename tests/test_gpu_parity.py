@@ -505,6 +505,28 @@ def test_conv_packed_residual(G, path, tile):
     assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
 
 
+@pytest.mark.parametrize("rbits", [3, 5, 8])
+@pytest.mark.parametrize("path,tile", [(0, None), (1, None), (1, 0), (2, 1), (2, 2), (2, 4), (2, 5), (2, 8), (3, 2), (4, 0),
+                                       (5, 1)])
+def test_conv_packed_residual_wide_codes(G, path, tile, rbits):
+    """Shortcut codes wider than two bits: their words are not staged before the K loop but read by the
+    output stage itself, one plane at a time."""
+    rng = np.random.default_rng(980 + path + 7 * (tile or 0) + rbits)
+    batch, H, Wd, C, wb, xb, ob = 2, 10, 12, 128, 1, 2, 2
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, C * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    acc = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw).reshape(-1, C)
+    short = rng.integers(0, 2 ** rbits, size=acc.shape).astype(np.uint32)
+    short_planes = O.pack_bits(short, acc.shape[0], C, C, rbits)
+    thr = np.sort(rng.integers(-150, 150, size=(C, 3)), axis=1).astype(np.int32)
+    d_thr, d_sp = G.to_dev(thr), G.to_dev(short_planes)
+    epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, resid_planes=d_sp, resid_bits=rbits, resid_scale=3)
+    got = G.run_conv(Wt, X, cin_pad=C, sym=1, epi=epi, path=path, tile=tile, **kw).view(np.uint32).reshape(ob, -1, C // 32)
+    q = O.bn_quantize(acc + 3 * short.astype(np.int32), None, thr, None, ob)
+    assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
+
+
 @pytest.mark.parametrize("R,stride,pad,H,Wd,cout,C", [
     (7, 2, 3, 40, 43, 64, 3), (11, 4, 5, 67, 70, 64, 3), (3, 1, 1, 9, 12, 96, 4), (5, 2, 2, 33, 36, 32, 1),
     # row length a multiple of 4 bytes: the kernel that consumes image rows as bytes
