@@ -531,7 +531,9 @@ def test_conv_packed_residual_wide_codes(G, path, tile, rbits):
     (7, 2, 3, 40, 43, 64, 3), (11, 4, 5, 67, 70, 64, 3), (3, 1, 1, 9, 12, 96, 4), (5, 2, 2, 33, 36, 32, 1),
     # row length a multiple of 4 bytes: the kernel that consumes image rows as bytes
     (7, 2, 3, 40, 44, 64, 3), (7, 2, 3, 75, 132, 128, 3), (11, 4, 5, 67, 72, 64, 3), (3, 2, 0, 20, 70, 32, 2),
-    (7, 4, 3, 39, 64, 64, 3)])
+    (7, 4, 3, 39, 64, 64, 3),
+    # a patch of more dwords than a lane keeps in flight (stride 13: 3 x 409 dwords): staged in place
+    (3, 13, 1, 40, 140, 32, 4)])
 def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, Wd, cout, C):
     """First layer with packed output, then max-pool on the bit-planes."""
     rng = np.random.default_rng(990 + R + Wd)
