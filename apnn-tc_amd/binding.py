@@ -63,7 +63,7 @@ DECLARED_SYMBOLS = _GEMM_NAMES + _CONV_NAMES + ["apnn_gemm", "apnn_conv", "apnn_
                                                 "apnn_conv_i8_bn_pack", "apnn_pool_planes", "apnn_quantize_pack", "apnn_fold_bn", "apnn_conv_pair",
                                                 "apnn_gemm_plan", "apnn_conv_plan", "apnn_quantize_pack_u8", "apnn_binarize_pack",
                                                 "apnn_residual_prepare",
-                                                "apnn_device_cus", "apnn_version"]
+                                                "apnn_device_error", "apnn_device_cus", "apnn_version"]
 
 
 class ApnnError(RuntimeError):
@@ -144,6 +144,8 @@ def lib():
         L.apnn_residual_prepare.restype = _ci
         L.apnn_fold_bn.argtypes = [_vp] * 4 + [ctypes.c_float] * 3 + [_ci, _ci, _vp, _vp]
         L.apnn_fold_bn.restype = _ci
+        L.apnn_device_error.argtypes = [ctypes.POINTER(_ci), _vp]
+        L.apnn_device_error.restype = _ci
         L.apnn_device_cus.argtypes = []
         L.apnn_device_cus.restype = _ci
         L.apnn_version.argtypes = []

@@ -9,9 +9,35 @@
 #include "../../include/apnn_tc.h"
 #include "dispatch.h"
 
+// One error word per device (each device holds its own copy of a __device__ variable).
+__device__ int g_kernel_error_word;
+
 namespace {
 
 using apnn::KParams;
+
+constexpr int kMaxDevices = 64;
+std::atomic<int *> g_err_ptr[kMaxDevices];
+
+// Address of the current device's error word (nullptr if it cannot be obtained: kernels then skip the
+// report).  hipGetSymbolAddress once per device; the name of a __device__ variable is not a device
+// address in host code.
+int *kernel_error_word() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  int *ptr = g_err_ptr[dev].load(std::memory_order_acquire);
+  if (ptr != nullptr) return ptr;
+  void *sym = nullptr;
+  if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_kernel_error_word)) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g_err_ptr[dev].store(static_cast<int *>(sym), std::memory_order_release);
+  return static_cast<int *>(sym);
+}
 
 int check_dev_ptr(const void *p) {
   if (p == nullptr) return APNN_ENULL;
@@ -177,6 +203,22 @@ int epilogue_float_ok(const KParams &p, int wb, int xb) {
     sc = scale * ((1LL << p.resid_bits) - 1);
   }
   return acc + sc < (1LL << 24) ? 1 : 0;
+}
+
+// Every kernel accumulates (or, on the FP4 core, converts) into int32.  The largest magnitude a result
+// can take -- K x weight range x activation range, doubled by the symmetric-weight form 2*raw - wmax*sum,
+// plus the largest scaled shortcut code -- has to stay below 2^31; requests beyond that would wrap
+// silently and are refused.  (An int32 residual map adds a caller-supplied term that cannot be bounded
+// here; it wraps as int32 addition does.)
+bool int32_range_ok(long long kwords, int wb, int xb, bool sym, const apnn_epilogue &e) {
+  const long long span = ((1LL << wb) - 1) * ((1LL << xb) - 1);  // at most 255 * 255
+  long long top = kwords * 32 * span;                              // kwords <= 2^26 here: no overflow of int64
+  if (sym) top *= 2;
+  if (e.mode != APNN_EPI_INT32 && e.residual_planes != nullptr) {
+    const long long scale = e.residual_scale < 0 ? -(long long)e.residual_scale : e.residual_scale;
+    top += scale * ((1LL << e.residual_bits) - 1);
+  }
+  return top < (1LL << 31);
 }
 
 // Reports a kernel choice instead of launching it (apnn_gemm_plan / apnn_conv_plan).
@@ -419,6 +461,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   if ((d->path >> 16) != 0 || (path < APNN_PATH_AUTO || path > APNN_PATH_MFMA_XS))
     return APNN_EINVAL;
   if ((rc = check_epilogue(d->epi, d->N, false, 0, 0))) return rc;
+  if (!int32_range_ok(d->K / 32, d->wb, d->xb, d->weight_mode == APNN_WEIGHT_SYMMETRIC, d->epi)) return APNN_EINVAL;
 
   KParams p{};
   p.A = static_cast<const uint32_t *>(d->W);
@@ -513,6 +556,7 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   const int C32 = d->cin_pad / 32;
   const long long KW = (long long)d->R * d->S * C32;
   if (pixels > 0x7fffffffLL || KW > (1 << 20)) return APNN_EINVAL;
+  if (!int32_range_ok(KW, d->wb, d->xb, d->weight_mode == APNN_WEIGHT_SYMMETRIC, d->epi)) return APNN_EINVAL;
   // a chunk of 4 words must not straddle two taps when 128-bit loads are used
   const int vw = (C32 % 4 == 0) ? 4 : (C32 % 2 == 0) ? 2 : 1;
 
@@ -595,6 +639,7 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream, apnn_plan *plan = null
     const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
     if (pt >= 0) {
       p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
+      if (plan == nullptr) p.err = kernel_error_word();
       p.magicPW = magic_of(p.PWs);
       p.magicPH = magic_of(p.PHs);
       if (plan != nullptr)
@@ -908,6 +953,18 @@ int apnn_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const floa
   if (X == nullptr || Wt == nullptr || scale == nullptr || bias == nullptr || out == nullptr) return APNN_ENULL;
   if (B <= 0 || N <= 0 || K <= 0) return APNN_EINVAL;
   return (int)apnn::launch_fc_i8(X, Wt, scale, bias, out, acc_out, B, N, K, static_cast<hipStream_t>(s));
+}
+
+int apnn_device_error(int *code, apnn_stream_t s) {
+  if (code == nullptr) return APNN_ENULL;
+  *code = 0;
+  int *word = kernel_error_word();
+  if (word == nullptr) return APNN_EUNSUPPORTED;
+  hipStream_t stream = static_cast<hipStream_t>(s);
+  hipError_t e = hipStreamSynchronize(stream);
+  if (e == hipSuccess) e = hipMemcpy(code, word, sizeof(int), hipMemcpyDeviceToHost);
+  if (e == hipSuccess && *code != 0) e = hipMemset(word, 0, sizeof(int));
+  return (int)e;
 }
 
 int apnn_device_cus(void) { return device_cus(); }

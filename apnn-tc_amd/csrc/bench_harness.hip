@@ -123,6 +123,17 @@ int apnn_bench_gemm_graph(const apnn_gemm_desc *d, int warmup, int iters, int ba
   return timed_graph_loop([&](hipStream_t cs) { return apnn_gemm(d, cs); }, warmup, iters, batch, event_ms, wall_ms);
 }
 
+// Cold-cache variant: launch i works on descriptor descs[i % nsets], every descriptor naming buffers of
+// its own.  With graphs of `batch` = nsets launches and nsets x (bytes of one buffer set) larger than the
+// last-level cache, a buffer set is revisited only after every other set went through the caches.
+int apnn_bench_gemm_graph_rotate(const apnn_gemm_desc *descs, int nsets, int warmup, int iters, int batch,
+                                 float *event_ms, double *wall_ms) {
+  if (descs == nullptr || nsets < 1) return APNN_EINVAL;
+  long long next = 0;
+  return timed_graph_loop([&](hipStream_t cs) { return apnn_gemm(&descs[next++ % nsets], cs); }, warmup, iters, batch,
+                          event_ms, wall_ms);
+}
+
 // Runs `iters` back-to-back apnn_gemm launches of the same descriptor on `stream` after `warmup`
 // untimed ones.  event_ms: HIP-event time over the timed launches; wall_ms: host wall clock from
 // first launch to stream idle.
@@ -169,6 +180,32 @@ int apnn_bench_copy(const void *src, void *dst, long long bytes, apnn_stream_t s
   if (src == nullptr || dst == nullptr || bytes <= 0 || (bytes % 16) != 0) return APNN_EINVAL;
   hipLaunchKernelGGL(apnn_bench_copy_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(s),
                      static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), bytes / 16);
+  return (int)hipGetLastError();
+}
+
+// The int32 store of the matrix-core kernels, alone: a wave owns a 32-row x 32-column block and every
+// store instruction writes two 128-byte row segments (lane half g, register j -> row 8q + 4g + j,
+// lane%32 -> column), the segments of one instruction being four rows apart.  Writes rows x cols x 4
+// bytes exactly once; calibrates WRITE_SIZE for this store pattern.
+__global__ __launch_bounds__(256) void apnn_bench_store_blocks_kernel(int *__restrict__ dst, int rows, int cols) {
+  const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const int blocks_per_row = cols / 32;
+  const long long nblocks = (long long)(rows / 32) * blocks_per_row;
+  const long long wave0 = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  for (long long b = wave0; b < nblocks; b += (long long)gridDim.x * 4) {
+    const int r0 = (int)(b / blocks_per_row) * 32, c0 = (int)(b % blocks_per_row) * 32;
+    int *base = dst + (long long)(r0 + 4 * g) * cols + c0 + li;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) base[(long long)(8 * q + j) * cols] = (int)b + q + j;
+  }
+}
+
+int apnn_bench_store_blocks(int *dst, int rows, int cols, apnn_stream_t s) {
+  if (dst == nullptr || rows <= 0 || cols <= 0 || (rows % 32) != 0 || (cols % 32) != 0) return APNN_EINVAL;
+  hipLaunchKernelGGL(apnn_bench_store_blocks_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(s), dst, rows,
+                     cols);
   return (int)hipGetLastError();
 }
 

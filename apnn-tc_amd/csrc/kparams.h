@@ -70,6 +70,11 @@ struct KParams {
   int epi_float;
   void *out;
   long long out_plane;       // packed output: plane stride in words
+  // Device error word of the current device (see apnn_device_error in apnn_tc.h): a kernel that meets a
+  // launch it cannot serve ORs a KERR_* code into it before it leaves its tile unwritten.
+  int *err;
 };
+
+enum KernelError { KERR_PATCH_CAPACITY = 1 };
 
 }  // namespace apnn

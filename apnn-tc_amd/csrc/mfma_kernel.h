@@ -101,11 +101,19 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// old with lane LANE replaced by the wave-uniform value val (v_writelane_b32: one VALU operation)
-template <int LANE>
-__device__ __forceinline__ int write_lane(int val, int old) {
-  static_assert(LANE >= 0 && LANE < 64, "lane index");
-  asm("v_writelane_b32 %0, %1, %2" : "+v"(old) : "s"(val), "n"(LANE));
+// old with lanes LANE_LO / LANE_HI replaced by the wave-uniform values lo / hi (v_writelane_b32: one VALU
+// operation each).  A vector instruction that reads a scalar register written by the vector instruction
+// just before it (a compare mask) needs wait states that the compiler inserts only for instructions it
+// can see -- not for this opaque assembly -- so the block waits by itself (s_nop 1) and is safe whatever
+// produced its scalar sources.
+template <int LANE_LO, int LANE_HI>
+__device__ __forceinline__ int write_lane_pair(int lo, int hi, int old) {
+  static_assert(LANE_LO >= 0 && LANE_LO < 64 && LANE_HI >= 0 && LANE_HI < 64, "lane index");
+  asm("s_nop 1\n\t"
+      "v_writelane_b32 %0, %1, %3\n\t"
+      "v_writelane_b32 %0, %2, %4"
+      : "+v"(old)
+      : "s"(lo), "s"(hi), "n"(LANE_LO), "n"(LANE_HI));
   return old;
 }
 
@@ -261,15 +269,10 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
             constexpr int rlo = decltype(rlo_c)::value, rhi = decltype(rhi_c)::value;
             auto put = [&](auto slot_c, unsigned long long mask) {
               constexpr int slot = decltype(slot_c)::value;
-              // The bit reversal (channel c -> bit 31 - c%32) runs on the scalar unit, between the
-              // compare that produced the mask and the lane write that consumes it: a lane write (opaque
-              // assembly, which the compiler's hazard handling does not see) must not take its scalar
-              // source straight from a vector compare.
+              // bit reversal: channel c -> bit 31 - c%32 (scalar unit)
               const int lo = (int)__brev((uint32_t)mask), hi = (int)__brev((uint32_t)(mask >> 32));
-              int reg = (int)park[y][slot >> 1];
-              reg = write_lane<rlo + 32 * (slot & 1)>(lo, reg);
-              reg = write_lane<rhi + 32 * (slot & 1)>(hi, reg);
-              park[y][slot >> 1] = (uint32_t)reg;
+              park[y][slot >> 1] = (uint32_t)write_lane_pair<rlo + 32 * (slot & 1), rhi + 32 * (slot & 1)>(
+                  lo, hi, (int)park[y][slot >> 1]);
             };
             if constexpr (std::is_same<ValT, float>::value) {
               const bool hi1 = val >= Tf[y][1];

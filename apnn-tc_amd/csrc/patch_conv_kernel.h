@@ -76,7 +76,12 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
   const int q_lo = row_base(0);  // == (gy0*gst)*PWs + gx0*gst
   const int q_hi = row_base(last_row - a0) + (R - 1) * p.PWs + (p.S - 1);
   const int npp = q_hi - q_lo + 1;
-  if (npp > cap) return;  // the host sizes the patch for the worst tile; never taken
+  if (npp > cap) {
+    // The host sizes the patch for the worst tile, so this is never taken; if it ever were, the tile
+    // stays unwritten and the device error word says so instead of the launch looking successful.
+    if (tid == 0 && p.err != nullptr) atomicOr(p.err, (int)KERR_PATCH_CAPACITY);
+    return;
+  }
 
   // this lane's rows: patch-relative pixel index of row li of each of its FA row blocks
   int prow[FA];

@@ -306,6 +306,16 @@ int apnn_unpack_sum(const uint32_t *planes, int8_t *out, long long rows_out, int
 int apnn_fc_i8(const int8_t *X, const int8_t *Wt, const float *scale, const float *bias, float *out,
                int32_t *acc_out, int B, int N, int K, apnn_stream_t s);
 
+/* Device-side error report.  The reference's kernels have no error path at all (checkKernelErrors aborts
+ * on a failed launch only, APNN-TC-lib/bmmaTensorCoreGemm/src/71_bmmaTensorCoreGemm.cu:65-75); here a
+ * kernel that finds a launch it cannot serve (today: a tile of the patch-resident convolution whose input
+ * patch exceeds the capacity the host computed) leaves that tile unwritten and ORs a code into one error
+ * word per device.  This call waits for `stream`, copies the current device's word to *code (0 = no
+ * kernel reported anything since the last call) and clears it.  It synchronizes: call it where a
+ * host-side check of finished work belongs, not between launches of a latency-critical sequence. */
+#define APNN_DEVERR_PATCH_CAPACITY 1
+int apnn_device_error(int *code, apnn_stream_t stream);
+
 /* Library / device information: number of compute units of the current device (0 if none). */
 int apnn_device_cus(void);
 const char *apnn_version(void);

@@ -18,10 +18,41 @@ def to_dev(arr):
 
 
 def dev_empty_i32(n, fill=None):
-    t = torch.empty(int(n), dtype=torch.int32, device="cuda")
+    return guarded_empty(n, torch.int32, fill)
+
+
+GUARD_BYTES = 256         # either side of every output: keeps the 16-byte alignment the entry points ask for
+GUARD_BYTE = 0x5A
+_live_guards = []         # (whole buffer, payload bytes, what) of the outputs the running test allocated
+
+
+def guarded_empty(n, dtype=torch.int32, fill=None, what="output"):
+    """A device tensor of n elements with guard bytes before and after it.  check_guards() (run by
+    to_host() and after every GPU test) asserts that no guard byte changed, so a store next to an
+    output buffer fails the test that made it."""
+    nbytes = int(n) * torch.empty(0, dtype=dtype).element_size()
+    whole = torch.empty(nbytes + 2 * GUARD_BYTES, dtype=torch.uint8, device="cuda")
+    whole.fill_(GUARD_BYTE)
+    view = whole[GUARD_BYTES:GUARD_BYTES + nbytes].view(dtype)
     if fill is not None:
-        t.fill_(fill)
-    return t
+        view.fill_(fill)
+    _live_guards.append((whole, nbytes, what))
+    return view
+
+
+def check_guards(clear=False):
+    if not _live_guards:
+        return
+    torch.cuda.synchronize()
+    for whole, nbytes, what in _live_guards:
+        lo = whole[:GUARD_BYTES].cpu().numpy()
+        hi = whole[GUARD_BYTES + nbytes:].cpu().numpy()
+        assert (lo == GUARD_BYTE).all(), "store below the %s buffer (%d bytes): guard byte -%d changed" % (
+            what, nbytes, GUARD_BYTES - int(np.flatnonzero(lo != GUARD_BYTE)[-1]))
+        assert (hi == GUARD_BYTE).all(), "store past the %s buffer (%d bytes): guard byte +%d changed" % (
+            what, nbytes, int(np.flatnonzero(hi != GUARD_BYTE)[0]))
+    if clear:
+        _live_guards.clear()
 
 
 def ptr(t):
@@ -29,7 +60,7 @@ def ptr(t):
 
 
 def to_host(t, dtype=np.int32):
-    torch.cuda.synchronize()
+    check_guards()
     a = t.cpu().numpy()
     return a.view(dtype) if dtype != a.dtype else a
 

@@ -203,6 +203,50 @@ def test_fp4_accumulation_guard():
     assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4
 
 
+def test_int32_accumulator_range_guard():
+    """Results are int32: a request whose largest possible magnitude -- K x weight range x activation
+    range, doubled for symmetric weights, plus the largest scaled shortcut code -- reaches 2^31 would wrap
+    and is refused with APNN_EINVAL on every path, by the plan call and by the launching call alike."""
+    L = A.lib()
+    for wb, xb in [(8, 8), (4, 4), (2, 8), (1, 8)]:
+        span = (2 ** wb - 1) * (2 ** xb - 1)
+        k_ok = ((2 ** 31 - 1) // span) // 128 * 128
+        k_bad = k_ok + 128
+        assert k_ok * span < 2 ** 31 <= k_bad * span
+        for path in (A.PATH_AUTO, A.PATH_VALU):
+            rc, _ = _plan_gemm(M=64, N=64, K=k_ok, wb=wb, xb=xb, path=path)
+            assert rc == 0, (wb, xb, path)
+            rc, _ = _plan_gemm(M=64, N=64, K=k_bad, wb=wb, xb=xb, path=path)
+            assert rc == A.EINVAL, (wb, xb, path)
+        g = A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=64, N=64, K=k_bad, wb=wb, xb=xb)
+        assert L.apnn_gemm(ctypes.byref(g), None) == A.EINVAL
+        # symmetric weights double the range
+        k_sym = ((2 ** 31 - 1) // (2 * span)) // 128 * 128
+        rc, _ = _plan_gemm(M=64, N=64, K=k_sym, wb=wb, xb=xb, weight_mode=A.WEIGHT_SYMMETRIC)
+        assert rc == 0
+        rc, _ = _plan_gemm(M=64, N=64, K=k_sym + 128, wb=wb, xb=xb, weight_mode=A.WEIGHT_SYMMETRIC)
+        assert rc == A.EINVAL
+    # the w8a8 K = 131072 request (largest magnitude 8.5e9) that used to be accepted
+    rc, _ = _plan_gemm(M=64, N=64, K=131072, wb=8, xb=8)
+    assert rc == A.EINVAL
+    # a scaled shortcut code counts: w1a2, K = 1024 leaves room for 2^31 - 1 - 3072
+    epi = A.Epilogue(mode=A.EPI_BN, out_bits=2, thresholds=0x1000, residual_planes=0x1000, residual_bits=2)
+    epi.residual_scale = (2 ** 31 - 1 - 3072) // 3
+    rc, _ = _plan_gemm(M=64, N=64, K=1024, wb=1, xb=2, epi=epi)
+    assert rc == 0
+    epi.residual_scale += 1
+    rc, _ = _plan_gemm(M=64, N=64, K=1024, wb=1, xb=2, epi=epi)
+    assert rc == A.EINVAL
+    # convolution: 9 taps x 2^17 stored channels x 255 x 255 is far beyond; 9 x 128 x 255 x 255 is not
+    geo = dict(batch=1, H=8, Wd=8, COUT=64, R=3, S=3, stride=1, pad=1, halo=0, wb=8, xb=8)
+    rc, _ = _plan_conv(cin_pad=128, **geo)
+    assert rc == 0
+    rc, _ = _plan_conv(cin_pad=2 ** 17, **geo)
+    assert rc == A.EINVAL
+    c = A.ConvDesc(W=0x1000, X=0x1000, O=0x1000, cin_pad=2 ** 17, **geo)
+    assert L.apnn_conv(ctypes.byref(c), None) == A.EINVAL
+
+
 def test_plan_reports_the_dispatchers_choices():
     """Without a device the dispatcher assumes 256 compute units: the choices for the benchmark shapes."""
     rc, plan = _plan_gemm(M=64, N=1024, K=1024, wb=1, xb=2, path=A.PATH_AUTO)

@@ -399,7 +399,7 @@ def test_conv_i8_bn_and_pool_pack(G, R, stride, pad, H, cout):
     Ho = acc.shape[1]
     thr = np.sort(rng.integers(-60000, 60000, size=(cout, 3)), axis=1).astype(np.int32)
     dX, dW, dT = G.to_dev(X), G.to_dev(Wt), G.to_dev(thr)
-    d_codes = torch.empty(B * Ho * Ho * cout, dtype=torch.uint8, device="cuda")
+    d_codes = G.guarded_empty(B * Ho * Ho * cout, torch.uint8)
     d_acc = G.dev_empty_i32(B * Ho * Ho * cout, fill=-7)
     L = G.A.lib()
     G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, H, C, cout, R, R,
@@ -426,11 +426,11 @@ def test_unpack_sum_and_fc_i8(G):
     planes = O.pack_bits(codes, B * HW, C, cpad, bits)
     d_planes = G.to_dev(planes)
     L = G.A.lib()
-    d_un = torch.empty(B * HW * C, dtype=torch.int8, device="cuda")
+    d_un = G.guarded_empty(B * HW * C, torch.int8)
     G.A.check(L.apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_un), B * HW, 1, C, cpad, bits, 0, None), "unpack")
     torch.cuda.synchronize()
     assert np.array_equal(d_un.cpu().numpy().reshape(B * HW, C), codes.astype(np.int8))
-    d_pool = torch.empty(B * C, dtype=torch.int8, device="cuda")
+    d_pool = G.guarded_empty(B * C, torch.int8)
     G.A.check(L.apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_pool), B, HW, C, cpad, bits, 1, None), "pool")
     torch.cuda.synchronize()
     pooled = np.minimum(127, codes.reshape(B, HW, C).sum(1) >> 1).astype(np.int8)
@@ -438,7 +438,7 @@ def test_unpack_sum_and_fc_i8(G):
     Wt = rng.integers(-128, 128, size=(N, C)).astype(np.int8)
     scale = rng.uniform(0.001, 0.01, N).astype(np.float32)
     bias = rng.uniform(-1, 1, N).astype(np.float32)
-    d_out = torch.empty(B * N, dtype=torch.float32, device="cuda")
+    d_out = G.guarded_empty(B * N, torch.float32)
     d_acc = G.dev_empty_i32(B * N, fill=-7)
     dW, dS, dB = G.to_dev(Wt), torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
     G.A.check(L.apnn_fc_i8(G.ptr(d_pool), G.ptr(dW), G.ptr(dS), G.ptr(dB), G.ptr(d_out), G.ptr(d_acc), B, N, C, None), "fc")
@@ -460,7 +460,7 @@ def test_fc_i8_batches(G, Bn, N, K):
     Wt = rng.integers(-128, 128, size=(N, K)).astype(np.int8)
     scale = rng.uniform(0.001, 0.01, N).astype(np.float32)
     bias = rng.uniform(-1, 1, N).astype(np.float32)
-    d_out = torch.empty(Bn * N, dtype=torch.float32, device="cuda")
+    d_out = G.guarded_empty(Bn * N, torch.float32)
     d_acc = G.dev_empty_i32(Bn * N, fill=-7)
     dX, dW, dS, dB = G.to_dev(X), G.to_dev(Wt), torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda()
     G.A.check(G.A.lib().apnn_fc_i8(G.ptr(dX), G.ptr(dW), G.ptr(dS), G.ptr(dB), G.ptr(d_out), G.ptr(d_acc), Bn, N, K, None), "fc")
@@ -479,7 +479,7 @@ def test_unpack_sum_group_sizes(G, B, HW, C, cpad, bits, shift):
     rng = np.random.default_rng(960 + HW)
     codes = rng.integers(0, 1 << bits, size=(B * HW, C)).astype(np.uint32)
     d_planes = G.to_dev(O.pack_bits(codes, B * HW, C, cpad, bits))
-    d_pool = torch.empty(B * C, dtype=torch.int8, device="cuda")
+    d_pool = G.guarded_empty(B * C, torch.int8)
     G.A.check(G.A.lib().apnn_unpack_sum(G.ptr(d_planes), G.ptr(d_pool), B, HW, C, cpad, bits, shift, None), "pool")
     torch.cuda.synchronize()
     pooled = np.minimum(127, codes.reshape(B, HW, C).sum(1) >> shift).astype(np.int8)
@@ -553,7 +553,7 @@ def test_conv_i8_bn_pack_and_pool_planes(G, R, stride, pad, H, Wd, cout, C):
     expect = O.pack_bits(codes.reshape(rows, cout).astype(np.uint32), rows, cout, cout, bits)
     assert np.array_equal(G.to_host(d_planes, np.uint32).reshape(expect.shape), expect)
     # the uint8-code / int32 outputs of the same kernel
-    d_codes = torch.empty(rows * cout, dtype=torch.uint8, device="cuda")
+    d_codes = G.guarded_empty(rows * cout, torch.uint8)
     d_acc = G.dev_empty_i32(rows * cout, fill=-7)
     G.A.check(L.apnn_conv_i8_bn(G.ptr(dX), G.ptr(dW), G.ptr(dT), G.ptr(d_codes), G.ptr(d_acc), B, H, Wd, C, cout, R, R,
                                 stride, pad, bits, 128, None), "conv_i8_bn")
@@ -741,6 +741,82 @@ def test_fp4_guard_falls_back_to_int32_accumulation(G):
     got = G.run_gemm(Wr, X, M, N, K, 1, 4, path=0).reshape(M, N)
     pop = np.array([int(np.unpackbits(Wr[0, m].view(np.uint8)).sum()) for m in range(M)])
     assert np.array_equal(got, np.repeat((15 * pop)[:, None], N, axis=1))
+
+
+def test_device_error_word_stays_clear(G):
+    """apnn_device_error: after patch-resident convolutions on every tile shape (the only kernel that can
+    report: a patch larger than the capacity the host computed) the current device's error word reads 0,
+    and the results are the oracle's."""
+    rng = np.random.default_rng(77)
+    batch, H, Wd, C, cout = 3, 12, 10, 64, 128
+    X = O.random_planes(rng, 2, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, 1, cout * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=1, xb=2)
+    ref = O.conv(Wt, X, cwords=C // 32, sym_w=1, **kw)
+    code = ctypes.c_int(-1)
+    assert G.A.lib().apnn_device_error(ctypes.byref(code), None) == 0   # whatever earlier tests left
+    for tile in range(5):
+        got = G.run_conv(Wt, X, cin_pad=C, sym=1, path=G.A.PATH_MFMA_PATCH, tile=tile, **kw)
+        assert np.array_equal(got.reshape(ref.shape), ref), tile
+    code = ctypes.c_int(-1)
+    assert G.A.lib().apnn_device_error(ctypes.byref(code), None) == 0 and code.value == 0
+    assert G.A.lib().apnn_device_error(None, None) == G.A.ENULL
+
+
+@pytest.mark.parametrize("wb,xb", [(1, 2), (1, 3), (1, 4), (2, 2)])
+def test_fp4_exact_just_below_the_accumulation_limit(G, wb, xb):
+    """The FP4 matrix-core kernels accumulate in fp32 (raw / 4, exact while raw < 2^24).  At the largest
+    128-multiple K the host still admits (K * (2^w-1) * (2^a-1) just below 2^24) every way of summing on
+    that core has to be exact: a tile whose waves tile the output, a split-K tile (four partial fp32 sums
+    meet in LDS), the expand-while-staging kernel, with unsigned and symmetric weights -- on all-ones
+    operands (every output equals the closed form K * span, the largest value the guard admits) and on
+    random operands against the oracle.  The fp32 threshold compare of the quantizing epilogue is pinned
+    at the same magnitude with thresholds at K*span - 1, K*span, K*span + 1 and beyond 2^24."""
+    span = (2 ** wb - 1) * (2 ** xb - 1)
+    K = ((2 ** 24 - 1) // span) // 128 * 128
+    assert K * span < 2 ** 24 <= (K + 128) * span
+    M = N = 64
+    wmax = 2 ** wb - 1
+    ones_w = np.full((wb, M, K // 32), 0xFFFFFFFF, np.uint32)
+    ones_x = np.full((xb, N, K // 32), 0xFFFFFFFF, np.uint32)
+    rng = np.random.default_rng(2400 + 10 * wb + xb)
+    rand_w = O.random_planes(rng, wb, M, K // 32)
+    rand_x = O.random_planes(rng, xb, N, K // 32)
+    refs = {sym: O.gemm(rand_w, rand_x, M, N, K, wb, xb, sym_w=sym, nthreads=8) for sym in (0, 1)}
+    # path, pinned tile: 64x64 (waves tile the output), 32x32 split-K, expand-while-staging 64x64
+    variants = [(G.A.PATH_MFMA, 2), (G.A.PATH_MFMA, 4), (G.A.PATH_MFMA_XS, 2)]
+    for path, tile in variants:
+        plan = G.A.Plan()
+        d = G.A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=M, N=N, K=K, wb=wb, xb=xb, path=path | ((tile + 1) << 8))
+        assert G.A.lib().apnn_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.fp4_exact == 1
+        for sym in (0, 1):
+            got = G.run_gemm(ones_w, ones_x, M, N, K, wb, xb, sym=sym, path=path, tile=tile)
+            # all-ones weights are +wmax in both conventions: 2*K*span - wmax*K*(2^a-1) == K*span
+            assert np.all(got == K * span), (path, tile, sym, int(got.min()), int(got.max()))
+            got = G.run_gemm(rand_w, rand_x, M, N, K, wb, xb, sym=sym, path=path, tile=tile).reshape(M, N)
+            assert np.array_equal(got, refs[sym]), (path, tile, sym)
+    # quantizing epilogue, flip unset: thresholds around the one value every output takes
+    v = K * span
+    rows = {0: [v + 1, v + 2, 2 ** 24 + 5], 1: [v, v + 1, 2 ** 24 + 5], 2: [v - 1, v, 2 ** 24 + 5],
+            3: [-2 ** 24 - 5, v - 2, v]}
+    nt = 2 ** xb - 1
+    thr = np.zeros((N, nt), np.int64)
+    want_code = np.zeros(N, np.int64)
+    for c in range(N):
+        t3 = rows[c % 4]
+        # codes wider than two bits: pad with thresholds no value reaches
+        thr[c] = t3 + [2 ** 24 + 6 + k for k in range(nt - 3)]
+        want_code[c] = c % 4
+    thr = thr.astype(np.int32)
+    d_thr = G.to_dev(thr)
+    q = O.bn_quantize(np.full((M, N), v, np.int32), None, thr, None, xb)
+    assert np.array_equal(q, np.repeat(want_code[None, :], M, axis=0))
+    want = O.lowbits_pack(q, M, N, xb)
+    for path, tile in variants[:2]:
+        for sym in (0, 1):
+            epi = G.epilogue(mode=G.A.EPI_BN, out_bits=xb, thr=d_thr)
+            got = G.run_gemm(ones_w, ones_x, M, N, K, wb, xb, sym=sym, epi=epi, path=path, tile=tile)
+            assert np.array_equal(got.view(np.uint32).reshape(xb, M, N // 32), want), (path, tile, sym)
 
 
 @pytest.mark.parametrize("name,wb,xb,pack", [("apconv_w1a5", 1, 5, False), ("apconv_w2a6", 2, 6, False),
