@@ -37,7 +37,7 @@ INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA
 FP4_MFMA_PEAK_TOPS = 10100.0   # MI355X dense fp4 MFMA (the matrix-core path feeds 2-bit digits as e2m1 codes)
 # HBM bytes per launch of the headline kernel from the hardware counters (FETCH_SIZE 184.50 KiB x 2.0
 # calibration, WRITE_SIZE 256 KiB x 1.0): see profiles/gemm_w1a2_m64_n1024_k1024.md
-HEADLINE_TRAFFIC_BYTES = 639954
+HEADLINE_TRAFFIC_BYTES = 640000
 BASELINE_TOPS = 18.66          # reference README.md:142 (w1a2, M=64, N=K=1024, sm_86)
 GRAPH_BATCH = 200              # kernel launches per captured HIP graph
 MIN_TIMED_LAUNCHES = 2000      # the timed region of a latency-bound shape never holds fewer launches
