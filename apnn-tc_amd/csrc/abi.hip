@@ -134,6 +134,7 @@ valu_fn mfma_gemm_fn(int wb, int xb, bool i8) {
   if (wb == 1 && xb == 4) return i8 ? apnn::mfma_gemm_1_4_x : apnn::mfma4_gemm_1_4_x;
   if (wb == 2 && xb == 2) return i8 ? apnn::mfma_gemm_2_2_x : apnn::mfma4_gemm_2_2_x;
   if (i8) return nullptr;
+  if (wb == 1 && xb == 1) return apnn::mfma4_gemm_1_1_x;
   if (wb == 4 && xb == 4) return apnn::mfma4_gemm_4_4_x;
   if (wb == 1 && xb == 8) return apnn::mfma4_gemm_1_8_x;
   if (wb == 2 && xb == 8) return apnn::mfma4_gemm_2_8_x;
@@ -146,6 +147,8 @@ valu_fn mfma_conv_fn(int xb, int wb, bool i8) {
   if (xb == 4 && wb == 1) return i8 ? apnn::mfma_conv_4_1_x : apnn::mfma4_conv_4_1_x;
   if (xb == 2 && wb == 2) return i8 ? apnn::mfma_conv_2_2_x : apnn::mfma4_conv_2_2_x;
   if (i8) return nullptr;
+  if (xb == 5 && wb == 1) return apnn::mfma4_conv_5_1_x;
+  if (xb == 6 && wb == 2) return apnn::mfma4_conv_6_2_x;
   if (xb == 8 && wb == 1) return apnn::mfma4_conv_8_1_x;
   if (xb == 8 && wb == 2) return apnn::mfma4_conv_8_2_x;
   if (xb == 4 && wb == 4) return apnn::mfma4_conv_4_4_x;
@@ -219,6 +222,49 @@ bool int32_range_ok(long long kwords, int wb, int xb, bool sym, const apnn_epilo
     top += scale * ((1LL << e.residual_bits) - 1);
   }
   return top < (1LL << 31);
+}
+
+// resid_scale as terms the matrix cores can apply to FP4 shortcut digits (KParams::fold).  A digit v means
+// v / 2 and the accumulator holds result / vscale (vscale = 4, or 8 with symmetric weights), so a term
+// t = s * m * 2^j (m = 1 or 3) needs the FP4 value s * m / 2 (codes 1 and 3, sign in bit 3) and the block
+// scale 2^(j - sym).  Two terms at most; 0 when the scale needs more, when there is no packed shortcut of
+// one or two bits, or when fp32 could round (accumulator range plus both terms' largest magnitude must stay
+// below 2^24, as for epilogue_float_ok).
+uint32_t shortcut_fold(const KParams &p, int wb, int xb) {
+  if (p.resid_planes == nullptr || p.resid_bits < 1 || p.resid_bits > 2 || p.resid_scale == 0) return 0u;
+  if (p.epi == APNN_EPI_INT32 || p.pool != APNN_POOL_NONE) return 0u;
+  const long long S = p.resid_scale;
+  const int sym = p.sym ? 1 : 0;
+  auto term = [&](long long t, uint32_t *nib, uint32_t *e8) {  // t == +-{1,3} * 2^j with j >= 0?
+    if (t == 0) return false;
+    const long long a = t < 0 ? -t : t;
+    int j = 0;
+    long long m = a;
+    while ((m & 1) == 0) {
+      m >>= 1;
+      ++j;
+    }
+    if (m != 1 && m != 3) return false;
+    *nib = (m == 1 ? 1u : 3u) | (t < 0 ? 8u : 0u);
+    *e8 = (uint32_t)(127 + j - sym);
+    return true;
+  };
+  const long long acc = (long long)p.KW * 32 * ((1LL << wb) - 1) * ((1LL << xb) - 1);
+  const long long cmax = (1LL << p.resid_bits) - 1;
+  auto fits = [&](long long t0, long long t1) {
+    const long long a0 = t0 < 0 ? -t0 : t0, a1 = t1 < 0 ? -t1 : t1;
+    return acc + (a0 + a1) * cmax < (1LL << 24);
+  };
+  uint32_t n0 = 0, e0 = 127, n1 = 0, e1 = 127;
+  if (term(S, &n0, &e0)) return fits(S, 0) ? (n0 | (e0 << 8) | (127u << 16)) : 0u;
+  for (int j = 0; j < 24; ++j)
+    for (int m = 1; m <= 3; m += 2)
+      for (int sg = -1; sg <= 1; sg += 2) {
+        const long long t0 = (long long)sg * m * (1LL << j);
+        if (term(t0, &n0, &e0) && term(S - t0, &n1, &e1) && fits(t0, S - t0))
+          return n0 | (n1 << 4) | (e0 << 8) | (e1 << 16);
+      }
+  return 0u;
 }
 
 // Reports a kernel choice instead of launching it (apnn_gemm_plan / apnn_conv_plan).
@@ -321,7 +367,7 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
 int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3, bool int32_out = false) {
-  const bool wide = planes > 5;
+  const bool wide = planes > 5 || planes == 2;  // the reduced tile set (see mfma_tile_enabled)
   int cus = device_cus();
   if (cus <= 0) cus = 256;
   auto ntiles = [&](int t) {
@@ -332,7 +378,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
   auto fill = [&](int t) {
     return (double)rowsA * rowsB / ((double)ntiles(t) * apnn::kMfmaTileA[t] * apnn::kMfmaTileB[t]);
   };
-  if (wide) {  // more than five planes in all: 128x128, 64x64 and the 32x32 split-K tile are built
+  if (wide) {  // more than five planes in all, or w1a1: 128x128, 64x64 and the 32x32 split-K tile are built
     if (conv && vw != 4) return 2;
     if (KW >= 32 && ntiles(4) <= 256) return 4;
     return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
@@ -445,8 +491,9 @@ int plan_direct(apnn_plan *plan, const KParams &p, bool f4ok) {
 
 int plan_mfma(apnn_plan *plan, bool i8, int tile, const KParams &p, bool f4ok) {
   const bool split = tile == apnn::MT_32x32_K4 || tile == apnn::MT_32x64_K4 || tile == apnn::MT_32x128_K4;
+  const int ksplit = split ? 4 : (tile == apnn::MT_128x128_G2 ? 2 : 1);
   return fill_plan(plan, i8 ? APNN_PATH_MFMA_I8 : APNN_PATH_MFMA, i8 ? APNN_KERNEL_MFMA_I8 : APNN_KERNEL_MFMA_FP4, tile,
-                   apnn::kMfmaTileA[tile], apnn::kMfmaTileB[tile], split ? 4 : 1, p, 0, f4ok);
+                   apnn::kMfmaTileA[tile], apnn::kMfmaTileB[tile], ksplit, p, 0, f4ok);
 }
 
 // plan != nullptr: report the choice, launch nothing
@@ -480,6 +527,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   p.planesB = d->xb;
   const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
   p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
+  p.fold = shortcut_fold(p, d->wb, d->xb);
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
   if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_XS) && !f4ok) return APNN_EUNSUPPORTED;  // fp32 would round
   if (path == APNN_PATH_MFMA_XS) {
@@ -586,6 +634,7 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   p.planesA = d->xb;
   p.planesB = d->wb;
   p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
+  p.fold = shortcut_fold(p, d->wb, d->xb);
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;

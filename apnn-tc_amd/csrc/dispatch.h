@@ -32,6 +32,9 @@ APNN_DECL_MFMA(conv, 2, 1)
 APNN_DECL_MFMA(conv, 3, 1)
 APNN_DECL_MFMA(conv, 4, 1)
 APNN_DECL_MFMA(conv, 2, 2)
+APNN_DECL_MFMA4(gemm, 1, 1)
+APNN_DECL_MFMA4(conv, 5, 1)
+APNN_DECL_MFMA4(conv, 6, 2)
 APNN_DECL_MFMA4(gemm, 4, 4)
 APNN_DECL_MFMA4(gemm, 1, 8)
 APNN_DECL_MFMA4(gemm, 2, 8)
@@ -70,12 +73,14 @@ APNN_DECL_PATCH(2, 2)
 enum { CORE_I8 = 0, CORE_F4 = 1 };
 
 // tile shapes of the MFMA kernels, index = enum MfmaTile in mfma_kernel.h
-constexpr int kMfmaTileCount = 9;
-constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128, 32};
-constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256, 128};
+constexpr int kMfmaTileCount = 10;
+constexpr int kMfmaTileA[kMfmaTileCount] = {256, 128, 64, 128, 32, 32, 256, 128, 32, 128};
+constexpr int kMfmaTileB[kMfmaTileCount] = {256, 128, 64, 64, 32, 64, 128, 256, 128, 128};
 
+// MT_128x128_G2: the 128x128 tile computed by two groups of four waves that share its k-steps (work-groups
+// of 512 threads)
 enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_32x32_K4 = 4, MT_32x64_K4 = 5,
-                MT_256x128 = 6, MT_128x256 = 7, MT_32x128_K4 = 8, MT_COUNT = 9 };
+                MT_256x128 = 6, MT_128x256 = 7, MT_32x128_K4 = 8, MT_128x128_G2 = 9, MT_COUNT = 10 };
 
 // Which (core, family, load width, tile, plane counts) combinations are built.  Every kernel
 // instantiation costs seconds of compile time, so only the shapes the dispatcher can choose are kept:
@@ -87,7 +92,9 @@ enum MfmaTile { MT_256x256 = 0, MT_128x128 = 1, MT_64x64 = 2, MT_128x64 = 3, MT_
 //               more than five planes in all (w4a4, w1a8, w2a8): 128x128, 64x64, 32x32 split-K
 //               (convolution with narrower loads: 64x64 only); the int8 core is not built for those.
 constexpr bool mfma_tile_enabled(int core, bool conv, int vw, int tile, int pa, int pb) {
-  if (pa + pb > 5) {
+  // two wave groups: FP4 core, 128-bit loads, the four benchmark precisions
+  if (tile == MT_128x128_G2) return core == CORE_F4 && pa + pb <= 5 && pa + pb > 2 && (!conv || vw == 4);
+  if (pa + pb > 5 || pa + pb == 2) {
     if (core == CORE_I8) return false;
     if (conv && vw != 4) return tile == MT_64x64;
     return tile == MT_128x128 || tile == MT_64x64 || tile == MT_32x32_K4;

@@ -68,6 +68,11 @@ struct KParams {
   // 1: every value the quantizing epilogue compares (accumulator, correction, scaled shortcut code) is an
   // integer below 2^24 in magnitude, so the FP4 kernels may do the threshold compare in fp32
   int epi_float;
+  // Shortcut add on the matrix cores (FP4 kernels, see fold_shortcut in mfma_kernel.h): resid_scale as the
+  // sum of two terms +-{1, 3} * 2^j, each an FP4 value (sign and code in a nibble: bits 0-3 first term,
+  // bits 4-7 second term, 0 = no term) times an E8M0 block scale (bits 8-15 and 16-23).  0: the shortcut is
+  // added per value in the vector ALUs (scale not representable, fp32 would round, other core).
+  uint32_t fold;
   void *out;
   long long out_plane;       // packed output: plane stride in words
   // Device error word of the current device (see apnn_device_error in apnn_tc.h): a kernel that meets a

@@ -232,13 +232,13 @@ __device__ __forceinline__ void direct_epilogue(const KParams &p, AccT (&acc)[FA
               u[j] = __builtin_fmaf((float)acc[x][y][4 * q + j], vscale, CONV ? negcf[j] : cnegf[y]);
               v[j] = 0;
             } else {
-              int t;
               if constexpr (F4) {
-                t = (int)(acc[x][y][4 * q + j] * 4.0f);  // an integer already: truncation is exact
+                // acc * vscale is an integer already (also with a folded shortcut, which adds multiples
+                // of 1 / vscale): the conversion is exact
+                v[j] = (int)(acc[x][y][4 * q + j] * vscale) + (CONV ? negc[j] : cneg[y]);
               } else {
-                t = acc[x][y][4 * q + j];
+                v[j] = (acc[x][y][4 * q + j] << sh) + (CONV ? negc[j] : cneg[y]);
               }
-              v[j] = (t << sh) + (CONV ? negc[j] : cneg[y]);
               u[j] = 0.f;
             }
           });
@@ -499,6 +499,40 @@ __device__ __forceinline__ void wave_epilogue(const KParams &p, const int *slab,
   }
 }
 
+// Shortcut add on the matrix cores (FP4 core, shortcut codes of one or two bits).  The term
+// resid_scale * code[row][channel] of a 32x32 block is the product of the 32x32 matrix of codes (an FP4
+// operand like any activation row: digit v means v/2) with a scaled identity, so one more matrix
+// instruction per block adds it to the accumulator -- instead of two bit extracts, a merge, a multiply, a
+// conversion and an add per output value in the vector ALUs.  The scale travels as FP4 value x E8M0 block
+// scale; the two lane halves (k positions 0..31 and 32..63) both see the codes and carry one term each, so
+// resid_scale = t0 + t1 with t = +-{1, 3} * 2^j (the host finds the terms: KParams::fold, 0 when there
+// are none or fp32 would round).  res: the wave's published shortcut words, index
+// ((x * 2 + plane) * FB + y) * 32 + row.
+template <int FA, int FB>
+__device__ __forceinline__ void fold_shortcut(const KParams &p, v16f (&acc)[FA][FB], const uint32_t *res, int lane) {
+  const int li = lane & 31, g = lane >> 5;
+  const uint32_t nib = (p.fold >> (4 * g)) & 0xfu;
+  const uint32_t e8 = (p.fold >> (8 + 8 * g)) & 0xffu;
+  const int scale_b = (int)(e8 * 0x01010101u);
+  // identity column li: the shortcut planes hold channel c at bit 31 - c%32, and element e of a packed word
+  // is nibble e / 4 of operand word e % 4 (expand_fp4), so channel li pairs with element e = 31 - li
+  const int e = 31 - li;
+  const uint32_t one = nib << (4 * (e >> 2));
+  const v8i bop = {(e & 3) == 0 ? (int)one : 0, (e & 3) == 1 ? (int)one : 0, (e & 3) == 2 ? (int)one : 0,
+                   (e & 3) == 3 ? (int)one : 0, 0, 0, 0, 0};
+  static_for<0, FA>([&](auto xc) {
+    constexpr int x = decltype(xc)::value;
+    static_for<0, FB>([&](auto yc) {
+      constexpr int y = decltype(yc)::value;
+      uint32_t w[2];
+      w[0] = res[((x * 2 + 0) * FB + y) * 32 + li];
+      w[1] = p.resid_bits > 1 ? res[((x * 2 + 1) * FB + y) * 32 + li] : 0u;
+      const v8i aop = expand_fp4<2, 0>(w);
+      acc[x][y] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aop, bop, acc[x][y], 4, 4, 0, 0x7F7F7F7F, 0, scale_b);
+    });
+  });
+}
+
 // Epilogue operands a wave requests before its K loop and consumes after it.
 template <int FA, int FB>
 struct EpiOperands {
@@ -615,6 +649,17 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
           table[i] = gcol < p.rowsB ? p.thr[(long long)gcol * nt + k] : 0;
         }
       }
+      bool shortcut_vec = res_prefetched;
+      if constexpr (F4) {
+        if (res_prefetched && p.fold != 0u) {
+          // the shortcut term enters one of the partial sums (wave 0's) on the matrix cores
+          if (wave == 0) {
+            shortcut_publish<RES_REGS>(area + 32, lane, 64, res_regs[0]);
+            fold_shortcut<1, FB>(p, acc, area + 32, lane);
+          }
+          shortcut_vec = false;
+        }
+      }
       static_for<0, FB>([&](auto yc) {
         constexpr int y = decltype(yc)::value;
         static_for<0, 4>([&](auto qc) {
@@ -665,11 +710,11 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
         if constexpr (DIRECT_BITS > 2) {
           if (use_table) {
             direct_epilogue<F4, 1, FB, CONV, true, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm,
-                                                             res_prefetched, table);
+                                                             shortcut_vec, table);
             return;
           }
         }
-        direct_epilogue<F4, 1, FB, CONV, false, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm, res_prefetched);
+        direct_epilogue<F4, 1, FB, CONV, false, q, q + 1>(p, accr, stot, area, rb, cb, lane, thrT, flipm, shortcut_vec);
       };
       static_assert(KS == 4, "one register quad per wave");
       switch (wave) {
@@ -703,11 +748,20 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
 #pragma unroll
         for (int x = 0; x < FA; ++x) shortcut_publish<RES_REGS>(area + FA * 32 + x * 64 * FB, lane, 64, res_regs[x]);
       }
+      bool shortcut_vec = res_prefetched;  // shortcut still to be added per value by the vector ALUs
+      // (tiles of eight blocks per wave have no registers to spare for the extra operands)
+      if constexpr (F4 && FA * FB <= 4) {
+        if (res_prefetched && p.fold != 0u) {
+          // LDS operations of one wave complete in order: the words published above are visible here
+          fold_shortcut<FA, FB>(p, acc, area + FA * 32, lane);
+          shortcut_vec = false;
+        }
+      }
       const int rb = a0 + wa * FA * 32, cb = b0 + wb * FB * 32;
       if (DIRECT_BITS == 2 || p.out_bits <= 2) {
-        direct_epilogue<F4, FA, FB, CONV, false>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+        direct_epilogue<F4, FA, FB, CONV, false>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, shortcut_vec);
       } else if constexpr (DIRECT_BITS > 2) {
-        direct_epilogue<F4, FA, FB, CONV, true>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, res_prefetched);
+        direct_epilogue<F4, FA, FB, CONV, true>(p, acc, ssum, area, rb, cb, lane, thrT, flipm, shortcut_vec);
       }
       return;
     }
@@ -762,7 +816,8 @@ __device__ __forceinline__ void epi_finish(const KParams &p, AccT (&acc)[FA][FB]
 // for few outputs over a long K where every chunk iteration is a latency chain, stage 32: their per-chunk
 // work (im2col addressing, LDS staging, barrier) is a large share of a short K loop, and k-steps past the
 // end of K are skipped, so a longer chunk wastes nothing.
-constexpr int mfma_chunk_words(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
+constexpr int mfma_chunk_words(int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw, int ksx = 1) {
+  if (ksx > 1) return 16;  // two wave groups share the k-steps of a chunk: four each
   if (WA * WB == 1) return 32;
   if (conv && FA * FB <= 2 && vw == 4) return 16;
   if (!conv && FA * FB >= 8 && (PA * WA * FA + PB * WB * FB) * 32 <= 512) return 16;
@@ -772,8 +827,13 @@ constexpr int mfma_chunk_words(int PA, int PB, int FA, int FB, int WA, int WB, b
 // longest reduction (32-bit words) the one- and two-block convolution tiles load without staging
 constexpr int kDirectMaxKW = 40;
 
-template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC>
-__global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
+// KSX > 1: KSX groups of four waves each (work-groups of 256 * KSX threads).  Every group tiles the whole
+// output tile WA x WB like the four waves of the other kernels and takes every KSX-th k-step of each
+// staged chunk; after the K loop the groups exchange partial accumulators through LDS so that each group
+// finishes 1 / KSX of the tile's row blocks.  For layers with too few large tiles to give every compute
+// unit two work-groups: the second wave per SIMD comes from the same tile instead.
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC, int KSX = 1>
+__global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams pk) {
   // paired launch: the second half of the grid works on the second problem (see KParams)
   KParams p = pk;
   int bid = blockIdx.x;
@@ -794,14 +854,15 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   constexpr int KS = 4 / (WA * WB);
   static_assert(KS == 1 || FA == 1, "the split-K reduction handles one 32-row slab");
   constexpr bool F4 = CORE == CORE_F4;
+  static_assert(KSX == 1 || (KSX == 2 && KS == 1 && F4 && FA % 2 == 0), "wave groups: FP4 core, even row blocks");
   constexpr int WPS = F4 ? 2 : 1;                 // packed words per row consumed by one k-step
   constexpr int DA = F4 ? (PA + 1) / 2 : 1;       // operand digits (FP4: plane pairs)
   constexpr int DB = F4 ? (PB + 1) / 2 : 1;
   using AccT = typename std::conditional<F4, v16f, v16i>::type;
   using FragT = typename std::conditional<F4, v8i, v4i>::type;
-  constexpr int NT = 256;
+  constexpr int NT = 256 * KSX;
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr int KC = mfma_chunk_words(PA, PB, FA, FB, WA, WB, CONV, VW);
+  constexpr int KC = mfma_chunk_words(PA, PB, FA, FB, WA, WB, CONV, VW, KSX);
   constexpr int LD = KC + 1;         // odd row pitch: 32 rows hit 32 different banks
   constexpr int KQ = KC / VW;
   constexpr int UA = TA * KQ, UB = TB * KQ;
@@ -813,7 +874,9 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 31, g = lane >> 5;
-  const int wa = KS > 1 ? 0 : wave / WB, wb = KS > 1 ? 0 : wave % WB;
+  const int kq = KSX > 1 ? wave >> 2 : 0;   // wave group
+  const int wv = KSX > 1 ? wave & 3 : wave; // wave within its group
+  const int wa = KS > 1 ? 0 : wv / WB, wb = KS > 1 ? 0 : wv % WB;
 
   const int tilesB = (p.rowsB + TB - 1) / TB;
   const int a0 = (bid / tilesB) * TA;
@@ -852,7 +915,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
 
   // how the operands reach the matrix core (see direct_loop below)
   constexpr bool DIRECT_K = F4 && KS > 1 && VW == 4;
-  constexpr bool DIRECT_OPT = F4 && CONV && KS == 1 && FA == 1 && FB <= 2;
+  constexpr bool DIRECT_OPT = F4 && CONV && KS == 1 && KSX == 1 && FA == 1 && FB <= 2;
   const bool direct_k = DIRECT_OPT && p.KW <= kDirectMaxKW;
 
   // Operands from global memory straight into the registers the matrix core reads -- no LDS staging, no
@@ -1024,9 +1087,11 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   for (int pl = 0; pl < PB; ++pl) rotB[pl] = (uint32_t)(4 * g - pl) & 31u;
 
   // quantizer and shortcut words of this wave's tile: requested now, consumed after the K loop
-  EpiOperands<FA, FB> eo;
-  constexpr bool EPI_LAZY = FA * FB >= 8;
-  epi_prefetch<KS, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, a0 + wa * FA * 32, b0 + wb * FB * 32, lane, eo);
+  constexpr int HA = FA / KSX;  // row blocks of the wave tile this wave finishes
+  const int own_rbase = a0 + (wa * FA + kq * HA) * 32;
+  EpiOperands<HA, FB> eo;
+  constexpr bool EPI_LAZY = HA * FB >= 8;
+  epi_prefetch<KS, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, own_rbase, b0 + wb * FB * 32, lane, eo);
 
   // packed words of this lane's rows for one k-step
   uint32_t wA[FA][PA], wB[FB][PB];
@@ -1138,7 +1203,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
   if (nchunks > 1) fetch(KC);
   __syncthreads();
   if constexpr (KS == 1) {
-    read_words(smem, 0);
+    read_words(smem, kq);
     expand_all(af, bf);
   }
   for (int ch = 0; ch < nchunks; ++ch) {
@@ -1177,6 +1242,21 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
         __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);  // then its share of VALU work
       }
     };
+    if constexpr (KSX > 1) {
+      // wave group kq owns k-steps kq, kq + KSX, ... of every chunk (steps past the end of K read the
+      // zeros the staging wrote there)
+#pragma unroll 1
+      for (int ks = kq; ks + KSX < NKS; ks += KSX) {
+        read_words(cur, ks + KSX);
+        mfma_all();
+        advance();
+      }
+      __syncthreads();
+      if (more) read_words(nxt, kq);
+      mfma_all();
+      if (more) advance();
+      continue;
+    }
     // k-steps of this chunk that hold data (the last chunk may be short)
     const int nks = min(NKS, (p.KW - ch * KC + WPS - 1) / WPS);
     // k-steps 0 .. nks-2 (kept as a real loop: one scheduling region per k-step)
@@ -1203,11 +1283,75 @@ __global__ __launch_bounds__(256, OCC) void apnn_mfma_kernel(const KParams pk) {
     ssum[x] = t;
   }
 
-  epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
+  if constexpr (KSX == 1) {
+    epi_finish<F4, KS, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, acc, ssum, smem, wave, lane, a0, b0, wa, wb, eo);
+  } else {
+    // The two wave groups hold partial sums over their k-steps for the same outputs.  Group 0 finishes the
+    // first HA row blocks of every wave tile, group 1 the last HA: each wave parks the blocks it gives away
+    // in LDS in the accumulator's own register layout (16 bytes per lane and register quad), its partner
+    // (same position in the other group) adds them to its own.  Activation sums travel the same way.
+    static_assert(KSX == 2, "two wave groups");
+    __syncthreads();  // every wave is done with the staging buffers
+    float4 *xch = reinterpret_cast<float4 *>(smem);                  // [8 waves][HA][FB][4 quads][64 lanes]
+    int *xsum = reinterpret_cast<int *>(smem) + 8 * HA * FB * 4 * 64 * 4;  // [8 waves][FS][64 lanes]
+    auto give = [&](auto first_c) {
+      constexpr int first = decltype(first_c)::value;
+      static_for<0, HA>([&](auto xc) {
+        constexpr int x = decltype(xc)::value;
+        static_for<0, FB>([&](auto yc) {
+          constexpr int y = decltype(yc)::value;
+          static_for<0, 4>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            float4 v;
+            v.x = acc[first + x][y][4 * q];
+            v.y = acc[first + x][y][4 * q + 1];
+            v.z = acc[first + x][y][4 * q + 2];
+            v.w = acc[first + x][y][4 * q + 3];
+            xch[(((wave * HA + x) * FB + y) * 4 + q) * 64 + lane] = v;
+          });
+        });
+      });
+    };
+    if (kq == 0) give(std::integral_constant<int, HA>{}); else give(std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int x = 0; x < FS; ++x) xsum[(wave * FS + x) * 64 + lane] = ssum[x];
+    __syncthreads();
+    const int partner = wave ^ 4;
+    AccT own[HA][FB];
+    auto take = [&](auto first_c) {
+      constexpr int first = decltype(first_c)::value;
+      static_for<0, HA>([&](auto xc) {
+        constexpr int x = decltype(xc)::value;
+        static_for<0, FB>([&](auto yc) {
+          constexpr int y = decltype(yc)::value;
+          static_for<0, 4>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            const float4 v = xch[(((partner * HA + x) * FB + y) * 4 + q) * 64 + lane];
+            own[x][y][4 * q] = acc[first + x][y][4 * q] + v.x;
+            own[x][y][4 * q + 1] = acc[first + x][y][4 * q + 1] + v.y;
+            own[x][y][4 * q + 2] = acc[first + x][y][4 * q + 2] + v.z;
+            own[x][y][4 * q + 3] = acc[first + x][y][4 * q + 3] + v.w;
+          });
+        });
+      });
+    };
+    if (kq == 0) take(std::integral_constant<int, 0>{}); else take(std::integral_constant<int, HA>{});
+    int own_sum[CONV ? HA : FB];
+#pragma unroll
+    for (int x = 0; x < (CONV ? HA : FB); ++x) {
+      // convolution: sums of this group's row blocks; GEMM entry points: column sums, the same blocks in both groups
+      const int idx = CONV ? kq * HA + x : x;
+      own_sum[x] = xsum[(wave * FS + idx) * 64 + lane] + xsum[(partner * FS + idx) * 64 + lane];
+    }
+    // epi_finish opens with a barrier: nobody overwrites the exchange area before every wave has read it
+    epi_finish<F4, 1, CONV, (CONV ? PA : PB) >= 3 ? 4 : 2, EPI_LAZY>(p, own, own_sum, smem, wave, lane, own_rbase, b0, 0,
+                                                                       wb, eo);
+  }
 }
 
-constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw) {
-  const size_t ld = mfma_chunk_words(PA, PB, FA, FB, WA, WB, conv, vw) + 1;
+constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int WA, int WB, bool conv, int vw,
+                                 int ksx = 1) {
+  const size_t ld = mfma_chunk_words(PA, PB, FA, FB, WA, WB, conv, vw, ksx) + 1;
   // FP4 split-K tiles with 128-bit loads stage nothing (operands go from global memory to registers)
   const size_t stage = core == CORE_F4 && WA * WB == 1 && vw == 4
                            ? 0
@@ -1215,19 +1359,23 @@ constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int W
   // split-K tiles whose activations have three or more planes quantize codes of up to four bits from
   // registers and keep one threshold table [15][FB * 32] behind the output stage's area
   const size_t table = (WA * WB == 1 && (conv ? PA : PB) >= 3) ? 15ull * FB * 32 * sizeof(int) : 0;
-  const size_t slab = 4ull * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int) + table;
-  return stage > slab ? stage : slab;
+  const size_t slab = 4ull * ksx * (32 * (FB * 32 + 1) + 32 + FB * 32 + 2 * 32 * FB) * sizeof(int) + table;
+  // wave groups: exchange area of the partial accumulators and activation sums (see the kernel's tail)
+  const size_t fs = conv ? FA : FB;
+  const size_t xch = ksx > 1 ? 4ull * ksx * ((size_t)(FA / ksx) * FB * 16 + fs) * 64 * sizeof(int) : 0;
+  const size_t m = stage > slab ? stage : slab;
+  return m > xch ? m : xch;
 }
 
 // OCC_WANTED work-groups per compute unit, or as many as the LDS budget (160 KiB) allows
-template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED>
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED, int KSX = 1>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
-  constexpr size_t smem_bytes = mfma_smem_bytes(CORE, PA, PB, FA, FB, WA, WB, CONV, VW);
+  constexpr size_t smem_bytes = mfma_smem_bytes(CORE, PA, PB, FA, FB, WA, WB, CONV, VW, KSX);
   constexpr int OCC_FIT = (int)((160 * 1024) / smem_bytes);
   constexpr int OCC = OCC_FIT < 1 ? 1 : (OCC_FIT < OCC_WANTED ? OCC_FIT : OCC_WANTED);
   static_assert(smem_bytes * OCC <= 160 * 1024, "LDS budget of a gfx950 compute unit");
-  auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>;
+  auto kern = apnn_mfma_kernel<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC, KSX>;
   if (smem_bytes > 64 * 1024) {
     static bool raised = false;  // per instantiation; a repeated call is harmless
     if (!raised) {
@@ -1240,14 +1388,15 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   const long long tiles = (long long)((p.rowsA + TA - 1) / TA) * ((p.rowsB + TB - 1) / TB);
   KParams q = p;
   if (p.pair_tiles != 0) q.pair_tiles = (int)tiles;  // the host only flags a pair; the tile count is known here
-  hipLaunchKernelGGL(kern, dim3((unsigned)(q.pair_tiles != 0 ? 2 * tiles : tiles)), dim3(256), smem_bytes, stream, q);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(q.pair_tiles != 0 ? 2 * tiles : tiles)), dim3(256 * KSX), smem_bytes, stream,
+                     q);
   return hipGetLastError();
 }
 
-template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC, int TILE>
+template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC, int TILE, int KSX = 1>
 inline hipError_t launch_mfma_if_enabled(const KParams &p, hipStream_t stream) {
   if constexpr (mfma_tile_enabled(CORE, CONV, VW, TILE, PA, PB)) {
-    return launch_mfma<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC>(p, stream);
+    return launch_mfma<CORE, PA, PB, FA, FB, WA, WB, VW, CONV, OCC, KSX>(p, stream);
   } else {
     return hipErrorNotSupported;
   }
@@ -1265,6 +1414,7 @@ inline hipError_t launch_mfma_tile(int tile, const KParams &p, hipStream_t strea
     case MT_32x128_K4: return launch_mfma_if_enabled<CORE, PA, PB, 1, 4, 1, 1, VW, CONV, 2, MT_32x128_K4>(p, stream);
     case MT_256x128: return launch_mfma_if_enabled<CORE, PA, PB, 4, 2, 2, 2, VW, CONV, 2, MT_256x128>(p, stream);
     case MT_128x256: return launch_mfma_if_enabled<CORE, PA, PB, 2, 4, 2, 2, VW, CONV, 2, MT_128x256>(p, stream);
+    case MT_128x128_G2: return launch_mfma_if_enabled<CORE, PA, PB, 2, 2, 2, 2, VW, CONV, 1, MT_128x128_G2, 2>(p, stream);
     default: return hipErrorNotSupported;
   }
 }

@@ -94,7 +94,7 @@ def crossover_table(A, G, O, benchlib, stream):
 
     L = A.lib()
     out = []
-    gemm_cands = ([(A.PATH_VALU, t) for t in range(5)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 6)] +
+    gemm_cands = ([(A.PATH_VALU, t) for t in range(5)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 6, 9)] +
                   [(A.PATH_MFMA_I8, t) for t in (1, 2, 6)] + [(A.PATH_MFMA_XS, t) for t in (1, 2, 3, 6)])
     for (wb, xb, M, N, K) in [(1, 2, 64, 1024, 1024), (1, 4, 64, 1024, 1024), (1, 2, 128, 128, 2048), (1, 2, 256, 256, 1024),
                               (1, 2, 256, 256, 4096), (1, 2, 512, 512, 1024), (1, 2, 1024, 1024, 1024),
@@ -107,7 +107,7 @@ def crossover_table(A, G, O, benchlib, stream):
         cands = [c for c in gemm_cands if not (c[0] == A.PATH_VALU and M * N > 1024 * 1024 and c[1] != 0)]
         out.append(sweep("gemm w%da%d %dx%dx%d" % (wb, xb, M, N, K), d, L.apnn_gemm_plan, benchlib.apnn_bench_gemm_graph,
                          benchlib.apnn_bench_gemm, M * N <= 512 * 512, cands))
-    conv_cands = ([(A.PATH_VALU, t) for t in range(4)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 7, 8)] +
+    conv_cands = ([(A.PATH_VALU, t) for t in range(4)] + [(A.PATH_MFMA, t) for t in (1, 2, 3, 4, 5, 7, 8, 9)] +
                   [(A.PATH_MFMA_I8, t) for t in (1, 2, 3, 4, 7)] + [(A.PATH_MFMA_PATCH, t) for t in range(5)] +
                   [(A.PATH_MFMA_XS, t) for t in (1, 2, 3, 7)])
     geoms = [("conv16 b1 C=%d" % c, 1, 16, c, c, 3, 1, 1) for c in (128, 512, 1024)]

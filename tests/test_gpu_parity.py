@@ -59,9 +59,9 @@ CONV_PATHS_128 = CONV_PATHS + [5]   # shapes whose stored channel count is a mul
 # (path, pinned tile) pairs that are built: VALU tiles 0..3; FP4 GEMM all but 256x256 / 128x256;
 # int8 GEMM 128x128, 64x64, 256x128; FP4 convolution all but 256x256 / 256x128 (8 = 32x128 split-K); int8 convolution
 # 128x128, 64x64, 128x64, 32x32 split-K, 128x256
-GEMM_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)] +
+GEMM_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 6, 9)] + [(3, t) for t in (1, 2, 6)] +
               [(5, t) for t in (1, 2, 3, 6)])
-CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7, 8)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
+CONV_TILES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7, 8, 9)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
               [(4, t) for t in range(5)] + [(5, t) for t in (1, 2, 3, 7)])
 GEMM_TILES_PACKED = [pt for pt in GEMM_TILES if pt != (1, 3)]     # the VALU 16x16 tile has no packed epilogue
 CONV_TILES_PACKED = [pt for pt in CONV_TILES if pt != (1, 3)]
@@ -505,6 +505,35 @@ def test_conv_packed_residual(G, path, tile):
     assert np.array_equal(got, O.lowbits_pack(q, acc.shape[0], C, ob))
 
 
+@pytest.mark.parametrize("scale", [1, 3, 8, 7, 11, 21, -5, -12, 37, 1 << 14])
+@pytest.mark.parametrize("path,tile", [(0, None), (2, 1), (2, 2), (2, 3), (2, 4), (2, 5), (2, 8), (2, 9), (3, 2), (4, 0), (4, 3),
+                                       (5, 1)])
+def test_conv_packed_shortcut_scales(G, path, tile, scale):
+    """Shortcut codes of two bits and of one bit times an integer scale, added before the thresholds.  The FP4
+    kernels add the term on the matrix cores when the scale is a sum of two terms +-{1, 3} * 2^j (every
+    scale here but 37, which takes the per-value path like the other cores), symmetric and unsigned
+    weights, every kind of tile (waves tile the output, split K, two wave groups, patch-resident,
+    expanded while staging)."""
+    rng = np.random.default_rng(1980 + path + 7 * (tile or 0) + (scale & 1023))
+    batch, H, Wd, C, wb, xb, ob = 2, 10, 12, 128, 1, 2, 2
+    X = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+    Wt = O.random_planes(rng, wb, C * 9, C // 32)
+    kw = dict(batch=batch, H=H, W=Wd, cout=C, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+    for sym in (1, 0):
+        acc = O.conv(Wt, X, cwords=C // 32, sym_w=sym, **kw).reshape(-1, C)
+        for rbits in (2, 1):
+            short = rng.integers(0, 2 ** rbits, size=acc.shape).astype(np.uint32)
+            short_planes = O.pack_bits(short, acc.shape[0], C, C, rbits)
+            v = acc + scale * short.astype(np.int32)
+            lo, hi = int(v.min()), int(v.max())
+            thr = np.sort(rng.integers(lo, hi + 1, size=(C, 3)), axis=1).astype(np.int32)
+            d_thr, d_sp = G.to_dev(thr), G.to_dev(short_planes)
+            epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr, resid_planes=d_sp, resid_bits=rbits, resid_scale=scale)
+            got = G.run_conv(Wt, X, cin_pad=C, sym=sym, epi=epi, path=path, tile=tile, **kw)
+            q = O.bn_quantize(v, None, thr, None, ob)
+            assert np.array_equal(got.view(np.uint32).reshape(ob, -1, C // 32), O.lowbits_pack(q, acc.shape[0], C, ob)), (sym, rbits)
+
+
 @pytest.mark.parametrize("rbits", [3, 5, 8])
 @pytest.mark.parametrize("path,tile", [(0, None), (1, None), (1, 0), (2, 1), (2, 2), (2, 4), (2, 5), (2, 8), (3, 2), (4, 0),
                                        (5, 1)])
@@ -720,6 +749,43 @@ def test_wide_precisions_on_the_matrix_cores(G, wb, xb, tile, sym):
         Wn = O.random_planes(rng, wb, cout * 9, 2)
         nacc = O.conv(Wn, Xn, cwords=2, sym_w=sym, **kw)
         assert np.array_equal(G.run_conv(Wn, Xn, cin_pad=64, sym=sym, path=2, **kw).reshape(nacc.shape), nacc)
+
+
+@pytest.mark.parametrize("tile", [None, 1, 2, 4])
+@pytest.mark.parametrize("sym", [0, 1])
+def test_remaining_reference_precisions_on_the_matrix_cores(G, tile, sym):
+    """The reference tree's remaining precisions on the FP4 digit kernels: convolution w1a5 (three digits,
+    APNN-TC-lib/bmmaTensorCoreGemm/src/61_bmmaTensorCoreGemm.cu:58) and w2a6 (63_bmmaTensorCoreGemm.cu:58),
+    GEMM w1a1 (84_bmmaTensorCoreGemm.cu:80), int32 and quantized packed output, every tile that is built."""
+    rng = np.random.default_rng(6100 + 10 * (tile or 0) + sym)
+    M, N, K = 150, 200, 1152
+    W = O.random_planes(rng, 1, M, K // 32)
+    X = O.random_planes(rng, 1, N, K // 32)
+    acc = O.gemm(W, X, M, N, K, 1, 1, sym_w=sym, nthreads=8)
+    assert np.array_equal(G.run_gemm(W, X, M, N, K, 1, 1, sym=sym, path=2, tile=tile).reshape(M, N), acc)
+    plan = G.A.Plan()
+    d = G.A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=1024, N=1024, K=1024, wb=1, xb=1)
+    assert G.A.lib().apnn_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.kernel == G.A.KERNEL_MFMA_FP4
+    batch, H, Wd, C, cout = 2, 9, 10, 128, 96
+    for wb, xb in [(1, 5), (2, 6)]:
+        Xc = O.random_planes(rng, xb, batch * H * Wd, C // 32)
+        Wc = O.random_planes(rng, wb, cout * 9, C // 32)
+        kw = dict(batch=batch, H=H, W=Wd, cout=cout, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb)
+        cacc = O.conv(Wc, Xc, cwords=C // 32, sym_w=sym, nthreads=8, **kw)
+        got = G.run_conv(Wc, Xc, cin_pad=C, sym=sym, path=2, tile=tile, **kw)
+        assert np.array_equal(got.reshape(cacc.shape), cacc), (wb, xb)
+        rows = batch * H * Wd
+        for ob in (2, xb):
+            span = int(np.abs(cacc).max())
+            thr = np.sort(rng.integers(-span if sym else 0, span, size=(cout, 2 ** ob - 1)), axis=1).astype(np.int32)
+            d_thr = G.to_dev(thr)
+            epi = G.epilogue(mode=G.A.EPI_BN, out_bits=ob, thr=d_thr)
+            gotq = G.run_conv(Wc, Xc, cin_pad=C, sym=sym, epi=epi, path=2, tile=tile, **kw)
+            want = O.lowbits_pack(O.bn_quantize(cacc.reshape(rows, cout), None, thr, None, ob), rows, cout, ob)
+            assert np.array_equal(gotq.view(np.uint32).reshape(ob, rows, cout // 32), want), (wb, xb, ob)
+        c = G.A.ConvDesc(W=0x1000, X=0x1000, O=0x1000, batch=16, H=16, Wd=16, cin_pad=256, COUT=256, R=3, S=3, stride=1,
+                         pad=1, halo=1, wb=wb, xb=xb)
+        assert G.A.lib().apnn_conv_plan(ctypes.byref(c), ctypes.byref(plan)) == 0 and plan.kernel == G.A.KERNEL_MFMA_FP4
 
 
 def test_fp4_guard_falls_back_to_int32_accumulation(G):

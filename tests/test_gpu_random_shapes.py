@@ -21,9 +21,9 @@ def G():
     return gpu_util
 
 
-CONV_CHOICES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7, 8)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
+CONV_CHOICES = ([(1, t) for t in range(4)] + [(2, t) for t in (1, 2, 3, 4, 5, 7, 8, 9)] + [(3, t) for t in (1, 2, 3, 4, 7)] +
                 [(4, t) for t in range(5)] + [(5, t) for t in (1, 2, 3, 7)] + [(p, None) for p in (0, 0, 0, 1, 2, 3, 4, 5)])
-GEMM_CHOICES = ([(1, t) for t in range(5)] + [(2, t) for t in (1, 2, 3, 4, 5, 6)] + [(3, t) for t in (1, 2, 6)] +
+GEMM_CHOICES = ([(1, t) for t in range(5)] + [(2, t) for t in (1, 2, 3, 4, 5, 6, 9)] + [(3, t) for t in (1, 2, 6)] +
                 [(5, t) for t in (1, 2, 3, 6)] + [(p, None) for p in (0, 0, 0, 0, 1, 2, 3, 5)])
 CONV_COMBOS = [(1, 2), (1, 3), (1, 4), (2, 2)]
 GEMM_COMBOS = CONV_COMBOS + [(1, 8), (2, 8), (4, 4), (1, 1), (3, 5), (2, 1)]
