@@ -396,6 +396,16 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
     return (ntiles(1) >= cus && fill(1) >= 0.8) ? 1 : 2;
   }
   if (conv && vw == 1) return (ntiles(2) >= cus / 2 || KW < 16) ? 2 : 4;  // 32-bit loads: two tiles built
+  // About one 128x128 tile per compute unit over a long reduction (16x16 maps at batch 16 with 1024 channels,
+  // 14x14x256 at batch 64, 2048^2 outputs): plain 128x128 work-groups would leave one wave per SIMD, so two
+  // wave groups share each tile's k-steps.  Measured 11-18 % ahead of the best other tile there; with fewer
+  // tiles than that the idle compute units cost more than the split-K tiles' extra operand traffic
+  // (3/4 of the units busy against the 32x32 / 32x64 split-K tiles, 9/10 against 32x128).
+  if ((!conv || vw == 4) && planes > 2 && KW >= 64 && fill(1) >= 0.8) {
+    const long long nt1 = ntiles(1);
+    const bool wide_split_ok = conv && rowsB >= 512;  // the 32x128 split-K tile applies
+    if (2 * nt1 < 3 * cus && (wide_split_ok ? 10 * nt1 >= 9 * cus : 4 * nt1 >= 3 * cus)) return apnn::MT_128x128_G2;
+  }
   // Few outputs over a long reduction (batch-1 / batch-8 layers, 7x7 maps): the split-K tiles give
   // every 32x32 (32x64) block a work-group of its own and the four waves share K.  Measured
   // cross-overs on ResNet18 / 16x16 benchmark shapes.
@@ -528,6 +538,7 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
   const bool f4ok = fp4_exact(p.KW, d->wb, d->xb);
   p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
   p.fold = shortcut_fold(p, d->wb, d->xb);
+  p.addr32 = (unsigned long long)p.planeA * 4ull < (1ull << 32) && (unsigned long long)p.planeB * 4ull < (1ull << 32);
   if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;  // convolution only
   if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_XS) && !f4ok) return APNN_EUNSUPPORTED;  // fp32 would round
   if (path == APNN_PATH_MFMA_XS) {
@@ -541,7 +552,10 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
                        apnn::kMfmaTileB[tile], 1, p, 0, f4ok);
     return from_hip(fn(4, tile, p, stream));
   }
-  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma_gemm(p))) {
+  // operand planes of 4 GiB or more: the matrix-core kernels address rows with 32-bit offsets and refuse
+  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8) && !p.addr32) return APNN_EUNSUPPORTED;
+  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 ||
+      (path == APNN_PATH_AUTO && p.addr32 && auto_prefers_mfma_gemm(p))) {
     // AUTO: FP4 operands while their fp32 accumulation is exact, the int8 core (int32 accumulate) beyond
     const bool i8 = path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && !f4ok);
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, i8);
@@ -635,6 +649,16 @@ int build_conv_params(const apnn_conv_desc *d, KParams &p, int *vw_out) {
   p.planesB = d->wb;
   p.epi_float = epilogue_float_ok(p, d->wb, d->xb);
   p.fold = shortcut_fold(p, d->wb, d->xb);
+  {
+    const bool pow2 = (C32 & (C32 - 1)) == 0;
+    int sh = 0;
+    while ((1 << sh) < C32) ++sh;
+    const long long taps = (long long)d->R * d->S;
+    p.c32_shift = pow2 ? sh : -1;
+    p.magicS16 = (uint32_t)((65536 + d->S - 1) / d->S);
+    p.addr32 = taps * d->S < 65536 && (long long)p.Ws * d->R < (1 << 24) && C32 < (1 << 24) && KW < (1 << 24) &&
+               (unsigned long long)p.planeA * 4ull < (1ull << 32) && (unsigned long long)p.planeB * 4ull < (1ull << 32);
+  }
   p.batch = d->batch;
   p.PHs = d->H + 2 * d->pad;  // the padded frame: stored frame (incl. a stored halo) plus virtual padding
   p.PWs = d->Wd + 2 * d->pad;
@@ -698,7 +722,9 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream, apnn_plan *plan = null
     }
     if (path == APNN_PATH_MFMA_PATCH) return APNN_EUNSUPPORTED;
   }
-  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && auto_prefers_mfma(p))) {
+  // operand planes of 4 GiB or more, or a filter beyond the kernels' 24-bit index arithmetic: refused
+  if ((path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8) && !p.addr32) return APNN_EUNSUPPORTED;
+  if (path == APNN_PATH_MFMA || path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && p.addr32 && auto_prefers_mfma(p))) {
     const bool i8 = path == APNN_PATH_MFMA_I8 || (path == APNN_PATH_AUTO && !f4ok);
     valu_fn fn = mfma_conv_fn(d->xb, d->wb, i8);
     if (fn != nullptr) {
@@ -736,7 +762,7 @@ int run_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, hipStream_t 
   valu_fn fn = mfma_conv_fn(a->xb, a->wb, false);
   const bool fusable = fn != nullptr && plain_bn(a->epi) && plain_bn(b->epi) && a->epi.out_bits == b->epi.out_bits &&
                        (a->path & 0xffff) == APNN_PATH_AUTO && (b->path & 0xffff) == APNN_PATH_AUTO &&
-                       auto_prefers_mfma(pa) && a->O != b->O && fp4_exact(pa.KW, a->wb, a->xb) &&
+                       auto_prefers_mfma(pa) && pa.addr32 && pb.addr32 && a->O != b->O && fp4_exact(pa.KW, a->wb, a->xb) &&
                        fp4_exact(pb.KW, b->wb, b->xb);
   if (!fusable) {
     if ((rc = run_conv(a, stream))) return rc;

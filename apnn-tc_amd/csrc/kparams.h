@@ -39,6 +39,13 @@ struct KParams {
   // 1: every output row index times the larger of the row grid's sides stays below 2^32, so the
   // matrix-core kernels may decode a row index into (image, y, x) with magicGW / magicGH
   int geo_fast;
+  // 1: the matrix-core kernels of mfma_kernel.h may run: every operand plane spans less than 2^32 bytes
+  // (rows are addressed with 32-bit word offsets through buffer descriptors) and, for a convolution, the
+  // filter is small enough for 24-bit index arithmetic: taps * S < 65536, so that (tap * magicS16) >> 16 ==
+  // tap / S with magicS16 = ceil(65536 / S); stored width, C32 and KW below 2^24.
+  // c32_shift: log2(C32) when C32 is a power of two, else -1.
+  int addr32, c32_shift;
+  uint32_t magicS16;
 
   // Paired launch (matrix-core convolution kernels only): work-groups pair_tiles .. 2*pair_tiles-1
   // compute a second convolution on the same input and output grid (same A, rows, columns, stride,

@@ -872,7 +872,9 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   extern __shared__ __attribute__((aligned(16))) uint32_t smem[];  // [2][BUF_WORDS]
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  // the wave index is the same in all 64 lanes: as a scalar it keeps loop control and the address terms that
+  // depend on it (k-steps of a split-K wave, wave group) on the scalar unit
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 31, g = lane >> 5;
   const int kq = KSX > 1 ? wave >> 2 : 0;   // wave group
   const int wv = KSX > 1 ? wave & 3 : wave; // wave within its group
@@ -983,8 +985,14 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   }
 
   // ---- staging bookkeeping (same scheme as the VALU kernel) ----------------------------------
+  // The host launches this kernel only when every operand plane spans less than 2^32 bytes and the
+  // filter is small (KParams::addr32), so a row's chunk is addressed by a 32-bit word offset: the row's
+  // own offset, computed once, plus for a convolution a few full-rate operations per chunk -- tap =
+  // k / C32 (a shift when C32 is a power of two), (r, s) by multiply-shift, 24-bit multiplies -- instead of
+  // multiply-high decodes and 64-bit multiply-adds (quarter-rate operations) per chunk and row.
   int a_row[NIA], a_kq[NIA];
-  int a_b[NIA], a_y0[NIA], a_x0[NIA];
+  int a_y0[NIA], a_x0[NIA];
+  uint32_t a_base[NIA], b_base[NIB];  // word offset of the row (convolution: of the pixel's tap (0, 0), mod 2^32)
   bool a_ok[NIA];
   int b_row[NIB], b_kq[NIB];
   bool b_ok[NIB];
@@ -996,7 +1004,12 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
     a_row[it] = u / KQ;
     const int grow = a0 + a_row[it];
     a_ok[it] = (u < UA) && (grow < p.rowsA);
-    if (CONV) pixel_origin(grow, a_b[it], a_y0[it], a_x0[it]);
+    int ab = 0;
+    a_y0[it] = a_x0[it] = 0;
+    if (CONV) pixel_origin(grow, ab, a_y0[it], a_x0[it]);
+    a_base[it] = CONV ? (((uint32_t)ab * (uint32_t)p.Hs + (uint32_t)a_y0[it]) * (uint32_t)p.Ws + (uint32_t)a_x0[it]) *
+                            (uint32_t)p.C32
+                      : (uint32_t)grow * (uint32_t)p.KW;
   }
 #pragma unroll
   for (int it = 0; it < NIB; ++it) {
@@ -1004,42 +1017,77 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
     b_kq[it] = u % KQ;
     b_row[it] = u / KQ;
     b_ok[it] = (u < UB) && (b0 + b_row[it] < p.rowsB);
+    b_base[it] = (uint32_t)(b0 + b_row[it]) * (uint32_t)p.KW;
   }
   }
 
-  uint32_t ra_[NIA][PA][VW], rb_[NIB][PB][VW];
+  // Chunks in flight between global memory and LDS: the tiles of at most four blocks per wave keep two
+  // register sets, so a chunk's loads are issued two chunk iterations before they are staged (one iteration
+  // does not cover the memory latency when a wave runs only a few k-steps per chunk); the larger tiles have
+  // no registers to spare for a second set.
+  constexpr int PF = (FA * FB <= 4 && VW == 4) ? 2 : 1;
+  uint32_t ra_[PF][NIA][PA][VW], rb_[PF][NIB][PB][VW];
 
-  auto fetch = [&](int k0) {
+  // One buffer descriptor per operand plane (base, size in bytes).  A buffer load whose offset lies past
+  // the descriptor's size returns zeros, so a disabled load (row or k past the end, padding pixel) is the
+  // same instruction with the offset 0xffffffff: no branch around the load, which also lets the compiler
+  // count outstanding loads exactly (a register set waits for its own loads only).
+  __amdgpu_buffer_rsrc_t rsrcA[PA], rsrcB[PB];
+#pragma unroll
+  for (int pl = 0; pl < PA; ++pl)
+    rsrcA[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.A + pl * p.planeA), 0,
+                                                  (int)(uint32_t)(p.planeA * 4), 0x00020000);
+#pragma unroll
+  for (int pl = 0; pl < PB; ++pl)
+    rsrcB[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.B + pl * p.planeB), 0,
+                                                  (int)(uint32_t)(p.planeB * 4), 0x00020000);
+  auto load_buf = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t woff, bool ok, uint32_t (&dst)[VW]) {
+    const int boff = ok ? (int)(woff << 2) : -1;
+    if constexpr (VW == 4) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, boff, 0, 0);
+      dst[0] = v[0], dst[1] = v[1], dst[2] = v[2], dst[3] = v[3];
+    } else if constexpr (VW == 2) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, boff, 0, 0);
+      dst[0] = v[0], dst[1] = v[1];
+    } else {
+      dst[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff, 0, 0);
+    }
+  };
+
+  auto fetch = [&](int k0, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
 #pragma unroll
     for (int it = 0; it < NIA; ++it) {
       const int kw0 = k0 + a_kq[it] * VW;
       bool ok = a_ok[it] && kw0 < p.KW;
-      long long off;
+      uint32_t woff;
       if (CONV) {
-        const uint32_t tap = fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
-        const int cw = kw0 - (int)tap * p.C32;
-        const uint32_t r = fast_div(tap, (uint32_t)p.S, p.magicS);
-        const int s = (int)tap - (int)r * p.S;
-        const int iy = a_y0[it] + (int)r, ix = a_x0[it] + s;
-        ok = ok && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws;
-        off = (((long long)a_b[it] * p.Hs + iy) * p.Ws + ix) * p.C32 + cw;
+        const uint32_t tap = p.c32_shift >= 0 ? (uint32_t)kw0 >> p.c32_shift
+                                               : fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
+        const uint32_t cw = (uint32_t)kw0 - __umul24(tap, (uint32_t)p.C32);
+        const uint32_t r = __umul24(tap, p.magicS16) >> 16;
+        const uint32_t sx = tap - __umul24(r, (uint32_t)p.S);
+        const int iy = a_y0[it] + (int)r, ix = a_x0[it] + (int)sx;
+        ok = ok && (uint32_t)iy < (uint32_t)p.Hs && (uint32_t)ix < (uint32_t)p.Ws;
+        woff = a_base[it] + __umul24(__umul24(r, (uint32_t)p.Ws) + sx, (uint32_t)p.C32) + cw;
       } else {
-        off = (long long)(a0 + a_row[it]) * p.KW + kw0;
+        woff = a_base[it] + (uint32_t)kw0;
       }
 #pragma unroll
-      for (int pl = 0; pl < PA; ++pl) load_words<VW>(p.A + off + pl * p.planeA, ok, ra_[it][pl]);
+      for (int pl = 0; pl < PA; ++pl) load_buf(rsrcA[pl], woff, ok, ra_[set][it][pl]);
     }
 #pragma unroll
     for (int it = 0; it < NIB; ++it) {
       const int kw0 = k0 + b_kq[it] * VW;
       const bool ok = b_ok[it] && kw0 < p.KW;
-      const long long off = (long long)(b0 + b_row[it]) * p.KW + kw0;
+      const uint32_t woff = b_base[it] + (uint32_t)kw0;
 #pragma unroll
-      for (int pl = 0; pl < PB; ++pl) load_words<VW>(p.B + off + pl * p.planeB, ok, rb_[it][pl]);
+      for (int pl = 0; pl < PB; ++pl) load_buf(rsrcB[pl], woff, ok, rb_[set][it][pl]);
     }
   };
 
-  auto stage = [&](uint32_t *buf) {
+  auto stage = [&](uint32_t *buf, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
     uint32_t *As = buf;                   // [PA][TA][LD]
     uint32_t *Bs = buf + PA * TA * LD;    // [PB][TB][LD]
 #pragma unroll
@@ -1048,7 +1096,7 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
 #pragma unroll
         for (int pl = 0; pl < PA; ++pl)
 #pragma unroll
-          for (int i = 0; i < VW; ++i) As[(pl * TA + a_row[it]) * LD + a_kq[it] * VW + i] = ra_[it][pl][i];
+          for (int i = 0; i < VW; ++i) As[(pl * TA + a_row[it]) * LD + a_kq[it] * VW + i] = ra_[set][it][pl][i];
       }
     }
 #pragma unroll
@@ -1057,7 +1105,7 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
 #pragma unroll
         for (int pl = 0; pl < PB; ++pl)
 #pragma unroll
-          for (int i = 0; i < VW; ++i) Bs[(pl * TB + b_row[it]) * LD + b_kq[it] * VW + i] = rb_[it][pl][i];
+          for (int i = 0; i < VW; ++i) Bs[(pl * TB + b_row[it]) * LD + b_kq[it] * VW + i] = rb_[set][it][pl][i];
       }
     }
   };
@@ -1198,21 +1246,35 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
     if constexpr (DIRECT_OPT) direct_loop();
   } else {
   const int nchunks = (p.KW + KC - 1) / KC;
-  fetch(0);
-  stage(smem);
-  if (nchunks > 1) fetch(KC);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, PF - 1>;
+  // chunk c >= 1 travels in register set (c - 1) % PF
+  // (a fetch past the end of K is issued all the same, with every load disabled: the number of loads in
+  // flight is then the same on every path, and the compiler's wait counts stay exact)
+  fetch(0, Set0{});
+  stage(smem, Set0{});
+  if (PF == 2 || nchunks > 1) fetch(KC, Set0{});
+  if (PF == 2) fetch(2 * KC, Set1{});
   __syncthreads();
   if constexpr (KS == 1) {
     read_words(smem, kq);
     expand_all(af, bf);
   }
-  for (int ch = 0; ch < nchunks; ++ch) {
-    const uint32_t *cur = smem + (ch & 1) * BUF_WORDS;
-    uint32_t *nxt = smem + ((ch + 1) & 1) * BUF_WORDS;
+  // one chunk; par = ch % 2 is a compile-time constant (LDS buffer and register set of the iteration)
+  auto chunk_body = [&](int ch, auto par_c) {
+    const int par = par_c;
+    const uint32_t *cur = smem + par * BUF_WORDS;
+    uint32_t *nxt = smem + (par ^ 1) * BUF_WORDS;
     const bool more = ch + 1 < nchunks;
-    if (more) {
-      stage(nxt);  // every wave left this buffer before the barrier of the previous chunk
-      if (ch + 2 < nchunks) fetch((ch + 2) * KC);
+    // chunk ch + 1 leaves its registers (every wave left this LDS buffer before the barrier of the
+    // previous chunk), chunk ch + 1 + PF is requested into them
+    if constexpr (PF == 2) {
+      using Set = std::integral_constant<int, decltype(par_c)::value>;
+      if (more) stage(nxt, Set{});
+      fetch((ch + 3) * KC, Set{});
+    } else if (more) {
+      stage(nxt, Set0{});
+      if (ch + 2 < nchunks) fetch((ch + 2) * KC, Set0{});
     }
     if constexpr (KS > 1) {
       // split-K: wave w owns k-steps w, w + KS, ... of every chunk
@@ -1223,7 +1285,7 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
         mfma_all();
       }
       __syncthreads();
-      continue;
+      return;
     }
     auto advance = [&]() {
       FragT an[FA][DA], bn[FB][DB];
@@ -1255,7 +1317,7 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
       if (more) read_words(nxt, kq);
       mfma_all();
       if (more) advance();
-      continue;
+      return;
     }
     // k-steps of this chunk that hold data (the last chunk may be short)
     const int nks = min(NKS, (p.KW - ch * KC + WPS - 1) / WPS);
@@ -1271,6 +1333,20 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
     if (more) read_words(nxt, 0);
     mfma_all();
     if (more) advance();
+  };
+  if constexpr (PF == 2) {
+    // two chunks per trip: register set and LDS buffer of each half are compile-time constants (the only
+    // way back to the top is through both halves, so that the order of the loads in flight is the same on
+    // every path into the loop)
+#pragma unroll 1
+    for (int ch = 0;; ch += 2) {
+      chunk_body(ch, std::integral_constant<int, 0>{});
+      if (ch + 1 >= nchunks) break;
+      chunk_body(ch + 1, std::integral_constant<int, 1>{});
+      if (ch + 2 >= nchunks) break;
+    }
+  } else {
+    for (int ch = 0; ch < nchunks; ++ch) chunk_body(ch, ch & 1);
   }
   }
   int ssum[FS];
