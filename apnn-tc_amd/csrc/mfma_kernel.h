@@ -931,6 +931,32 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   //     the L1 cache, which costs less than the staging pipeline's bookkeeping for a handful of k-steps.
   // The first batch is requested here, before thresholds, shortcut words and accumulators are set up,
   // so that the rest of the prologue runs under its memory latency.
+  // One buffer descriptor per operand plane (base, size in bytes).  A buffer load whose offset lies past
+  // the descriptor's size returns zeros, so a disabled load (row or k past the end, padding pixel) is the
+  // same instruction with the offset 0xffffffff: no branch around the load, which also lets the compiler
+  // count outstanding loads exactly (a register set waits for its own loads only).
+  __amdgpu_buffer_rsrc_t rsrcA[PA], rsrcB[PB];
+#pragma unroll
+  for (int pl = 0; pl < PA; ++pl)
+    rsrcA[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.A + pl * p.planeA), 0,
+                                                  (int)(uint32_t)(p.planeA * 4), 0x00020000);
+#pragma unroll
+  for (int pl = 0; pl < PB; ++pl)
+    rsrcB[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.B + pl * p.planeB), 0,
+                                                  (int)(uint32_t)(p.planeB * 4), 0x00020000);
+  auto load_buf = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t woff, bool ok, uint32_t (&dst)[VW]) {
+    const int boff = ok ? (int)(woff << 2) : -1;
+    if constexpr (VW == 4) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, boff, 0, 0);
+      dst[0] = v[0], dst[1] = v[1], dst[2] = v[2], dst[3] = v[3];
+    } else if constexpr (VW == 2) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, boff, 0, 0);
+      dst[0] = v[0], dst[1] = v[1];
+    } else {
+      dst[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff, 0, 0);
+    }
+  };
+
   constexpr int GW = 2 * VW;
   constexpr int GD_BUDGET = KS > 1 ? (FB == 1 ? 60 : 48) : (FB == 1 ? 40 : 32);  // registers of operands in flight
   constexpr int GD_FIT = GD_BUDGET / (VW * (PA + FB * PB));
@@ -940,46 +966,52 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   const int ngroups = (p.KW + GW - 1) / GW;
   uint32_t ga[GD][PA][VW], gbw[GD][FB][PB][VW];
   bool okA = false;
-  int ab = 0, ay0 = 0, ax0 = 0;
-  const uint32_t *rowA = nullptr;
-  const uint32_t *rowB[FB];
+  int ay0 = 0, ax0 = 0;
+  uint32_t baseA = 0;  // word offset of this lane's row (convolution: of its pixel's tap (0, 0), mod 2^32)
+  uint32_t baseB[FB];
   bool okB[FB];
+  // Rows are addressed as in the staged path (32-bit word offsets, buffer loads that return zeros when
+  // disabled): the batch is straight-line code, so the wave starts on the first group while the loads of
+  // the later ones are still in flight.
   auto direct_issue = [&](int gb) {
 #pragma unroll
     for (int d = 0; d < GD; ++d) {
       const int kw0 = (gb + d * GSTEP) * GW + VW * g;
       const bool in_k = kw0 < p.KW;
       bool ok = okA && in_k;
-      const uint32_t *src;
+      uint32_t woff;
       if (CONV) {
-        const uint32_t tap = fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
-        const int cw = kw0 - (int)tap * p.C32;
-        const uint32_t r = fast_div(tap, (uint32_t)p.S, p.magicS);
-        const int s = (int)tap - (int)r * p.S;
-        const int iy = ay0 + (int)r, ix = ax0 + s;
-        ok = ok && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws;
-        src = p.A + ((((long long)ab * p.Hs + iy) * p.Ws + ix) * p.C32 + cw);
+        const uint32_t tap = p.c32_shift >= 0 ? (uint32_t)kw0 >> p.c32_shift
+                                               : fast_div((uint32_t)kw0, (uint32_t)p.C32, p.magicC32);
+        const uint32_t cw = (uint32_t)kw0 - __umul24(tap, (uint32_t)p.C32);
+        const uint32_t r = __umul24(tap, p.magicS16) >> 16;
+        const uint32_t sx = tap - __umul24(r, (uint32_t)p.S);
+        const int iy = ay0 + (int)r, ix = ax0 + (int)sx;
+        ok = ok && (uint32_t)iy < (uint32_t)p.Hs && (uint32_t)ix < (uint32_t)p.Ws;
+        woff = baseA + __umul24(__umul24(r, (uint32_t)p.Ws) + sx, (uint32_t)p.C32) + cw;
       } else {
-        src = rowA + kw0;
+        woff = baseA + (uint32_t)kw0;
       }
 #pragma unroll
-      for (int pl = 0; pl < PA; ++pl) load_words<VW>(src + pl * p.planeA, ok, ga[d][pl]);
+      for (int pl = 0; pl < PA; ++pl) load_buf(rsrcA[pl], woff, ok, ga[d][pl]);
 #pragma unroll
       for (int y = 0; y < FB; ++y)
 #pragma unroll
-        for (int pl = 0; pl < PB; ++pl) load_words<VW>(rowB[y] + kw0 + pl * p.planeB, okB[y] && in_k, gbw[d][y][pl]);
+        for (int pl = 0; pl < PB; ++pl) load_buf(rsrcB[pl], baseB[y] + (uint32_t)kw0, okB[y] && in_k, gbw[d][y][pl]);
     }
   };
   if (DIRECT_K || direct_k) {
     const int growA = a0 + wa * FA * 32 + li;
     okA = growA < p.rowsA;
+    int ab = 0;
     if (CONV) pixel_origin(growA, ab, ay0, ax0);
-    rowA = p.A + (long long)growA * p.KW;  // GEMM entry points
+    baseA = CONV ? (((uint32_t)ab * (uint32_t)p.Hs + (uint32_t)ay0) * (uint32_t)p.Ws + (uint32_t)ax0) * (uint32_t)p.C32
+                 : (uint32_t)growA * (uint32_t)p.KW;
 #pragma unroll
     for (int y = 0; y < FB; ++y) {
       const int grow = b0 + (wb * FB + y) * 32 + li;
       okB[y] = grow < p.rowsB;
-      rowB[y] = p.B + (long long)grow * p.KW;
+      baseB[y] = (uint32_t)grow * (uint32_t)p.KW;
     }
     direct_issue(gfirst);
   }
@@ -1027,32 +1059,6 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   // no registers to spare for a second set.
   constexpr int PF = (FA * FB <= 4 && VW == 4) ? 2 : 1;
   uint32_t ra_[PF][NIA][PA][VW], rb_[PF][NIB][PB][VW];
-
-  // One buffer descriptor per operand plane (base, size in bytes).  A buffer load whose offset lies past
-  // the descriptor's size returns zeros, so a disabled load (row or k past the end, padding pixel) is the
-  // same instruction with the offset 0xffffffff: no branch around the load, which also lets the compiler
-  // count outstanding loads exactly (a register set waits for its own loads only).
-  __amdgpu_buffer_rsrc_t rsrcA[PA], rsrcB[PB];
-#pragma unroll
-  for (int pl = 0; pl < PA; ++pl)
-    rsrcA[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.A + pl * p.planeA), 0,
-                                                  (int)(uint32_t)(p.planeA * 4), 0x00020000);
-#pragma unroll
-  for (int pl = 0; pl < PB; ++pl)
-    rsrcB[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.B + pl * p.planeB), 0,
-                                                  (int)(uint32_t)(p.planeB * 4), 0x00020000);
-  auto load_buf = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t woff, bool ok, uint32_t (&dst)[VW]) {
-    const int boff = ok ? (int)(woff << 2) : -1;
-    if constexpr (VW == 4) {
-      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, boff, 0, 0);
-      dst[0] = v[0], dst[1] = v[1], dst[2] = v[2], dst[3] = v[3];
-    } else if constexpr (VW == 2) {
-      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, boff, 0, 0);
-      dst[0] = v[0], dst[1] = v[1];
-    } else {
-      dst[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff, 0, 0);
-    }
-  };
 
   auto fetch = [&](int k0, auto set_c) {
     constexpr int set = decltype(set_c)::value;
