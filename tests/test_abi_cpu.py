@@ -247,6 +247,30 @@ def test_int32_accumulator_range_guard():
     assert L.apnn_conv(ctypes.byref(c), None) == A.EINVAL
 
 
+def test_matrix_core_kernels_refuse_operands_beyond_32_bit_offsets():
+    """The matrix-core kernels of the FP4 / int8 family address operand rows with 32-bit byte offsets
+    through buffer descriptors: a request whose operand plane reaches 4 GiB, or whose filter is beyond the
+    kernels' 24-bit index arithmetic, is refused when the family is pinned and served by the VALU kernels
+    (64-bit addressing) when the library chooses."""
+    # GEMM: one X plane of N x K / 8 bytes = 4 GiB
+    big = dict(M=256, N=1 << 17, K=1 << 18, wb=1, xb=2)
+    rc, plan = _plan_gemm(path=A.PATH_AUTO, **big)
+    assert rc == 0 and plan.kernel == A.KERNEL_VALU_TILE
+    for pinned in (A.PATH_MFMA, A.PATH_MFMA_I8):
+        rc, _ = _plan_gemm(path=pinned, **big)
+        assert rc == A.EUNSUPPORTED
+    rc, plan = _plan_gemm(path=A.PATH_AUTO, M=256, N=1 << 16, K=1 << 18, wb=1, xb=2)   # 2 GiB per plane
+    assert rc == 0 and plan.kernel in (A.KERNEL_MFMA_FP4, A.KERNEL_MFMA_I8)
+    # convolution: a 41 x 41 filter (taps * S >= 65536) is outside the multiply-shift tap decode
+    geo = dict(batch=4, H=64, Wd=64, cin_pad=128, COUT=256, stride=1, halo=0, wb=1, xb=2)
+    rc, plan = _plan_conv(R=41, S=41, pad=20, path=A.PATH_AUTO, **geo)
+    assert rc == 0 and plan.kernel == A.KERNEL_VALU_TILE
+    rc, _ = _plan_conv(R=41, S=41, pad=20, path=A.PATH_MFMA, **geo)
+    assert rc == A.EUNSUPPORTED
+    rc, plan = _plan_conv(R=11, S=11, pad=5, path=A.PATH_AUTO, **geo)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4
+
+
 def test_plan_reports_the_dispatchers_choices():
     """Without a device the dispatcher assumes 256 compute units: the choices for the benchmark shapes."""
     rc, plan = _plan_gemm(M=64, N=1024, K=1024, wb=1, xb=2, path=A.PATH_AUTO)
