@@ -366,7 +366,7 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3, bool int32_out = false) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3) {
   const bool wide = planes > 5 || planes == 2;  // the reduced tile set (see mfma_tile_enabled)
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -415,10 +415,12 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
     // compute unit (7x7x512 maps at batch 64, 16x16x512..1024 at batch 16): one activation expansion feeds
     // four blocks, 11-16 % faster than 32x64 / 128x64 there; with 256 channels or fewer tiles it loses
     if (vw == 4 && KW >= 64 && rowsB >= 512 && 2 * ntiles(8) >= 3 * cus && nb32 <= 4096) return 8;
-    // quantized output: up to two 32x32 work-groups per compute unit (measured 6-11 % ahead of 32x64 at 392
-    // and 512 blocks); int32 output, whose split-K store goes through LDS: at most one (32x64 is 10 % ahead
-    // at 512 blocks)
-    if (KW >= 32 && nb32 <= (int32_out ? 256 : 512)) return 4;
+    // 32x32 blocks, one work-group each: with three planes in all while every compute unit gets at most one
+    // (from 296 blocks the 32x64 tile, whose wave expands an activation block once for two channel blocks,
+    // is 5-9 % ahead with quantized output and level with int32 output); with four or more planes up to 2.5
+    // per compute unit (the second operand's expansion dominates and is not shared: 32x32 stays 2-12 %
+    // ahead up to 592 blocks, 32x64 takes over at 784).  Measured on 14x14x256 maps at batch 4..16.
+    if (KW >= 32 && nb32 <= (planes <= 3 ? 256 : 640)) return 4;
     if (KW >= 32 && nb32 <= 640) return 5;
     if (KW >= 64 && nb32 <= 3200) return 5;
   }
@@ -446,7 +448,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
 
 int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB, p.epi == APNN_EPI_INT32);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
@@ -561,16 +563,9 @@ int run_gemm(const apnn_gemm_desc *d, hipStream_t stream, apnn_plan *plan = null
     valu_fn fn = mfma_gemm_fn(d->wb, d->xb, i8);
     if (fn != nullptr) {
       if ((rc = pick_mfma_tile(tile_pin, p, false, 4, i8, &tile))) return rc;
-      // Four activation planes on the largest tile: the kernel that expands operands while staging reuses
-      // every 16-byte LDS operand for two digit pairs and measures 8 % faster at 8192^3 (w1a4); with fewer
-      // planes it is bound by LDS bandwidth and loses (see mfma_xs_kernel.h)
-      if (path == APNN_PATH_AUTO && !i8 && tile == apnn::MT_256x128 && d->wb == 1 && d->xb == 4) {
-        valu_fn xs = mfmaxs_gemm_fn(d->wb, d->xb);
-        if (plan != nullptr)
-          return fill_plan(plan, APNN_PATH_MFMA_XS, APNN_KERNEL_MFMA_FP4_XS, tile, apnn::kMfmaTileA[tile],
-                           apnn::kMfmaTileB[tile], 1, p, 0, f4ok);
-        return from_hip(xs(4, tile, p, stream));
-      }
+      // (The kernel that expands operands while staging, APNN_PATH_MFMA_XS, is never AUTO's choice: bound by
+      // LDS bandwidth, it measures 15-21 % behind this kernel on its best case, w1a4 at 4096^3..8192^3, and
+      // further behind with fewer planes -- see mfma_xs_kernel.h.)
       if (plan != nullptr) {
         // a pinned tile that is not built is reported by the launcher; mirror that here
         return apnn::mfma_tile_enabled(i8 ? apnn::CORE_I8 : apnn::CORE_F4, false, 4, tile, d->wb, d->xb)
@@ -709,7 +704,9 @@ int run_conv(const apnn_conv_desc *d, hipStream_t stream, apnn_plan *plan = null
   }
   if (path == APNN_PATH_MFMA_PATCH || (path == APNN_PATH_AUTO && f4ok)) {
     patch_fn pf = patch_conv_fn(d->xb, d->wb);
-    const int pt = pf == nullptr ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
+    // the kernel addresses pixels and filter rows by 32-bit byte offsets into each operand plane
+    const bool planes32 = (unsigned long long)p.planeA * 4ull < (1ull << 32) && (unsigned long long)p.planeB * 4ull < (1ull << 32);
+    const int pt = pf == nullptr || !planes32 ? -1 : choose_patch_tile(p, d->R, tile_pin, path == APNN_PATH_AUTO);
     if (pt >= 0) {
       p.patch_cap = patch_pixels(p, d->R, apnn::kPatchTileRows[pt]);
       if (plan == nullptr) p.err = kernel_error_word();
@@ -776,6 +773,7 @@ int run_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, hipStream_t 
   pa.S2 = pb.S;
   pa.pad2 = pb.pad;
   pa.magicS2 = pb.magicS;
+  pa.magicS16_2 = pb.magicS16;
   pa.planeB2 = pb.planeB;
   pa.thr2 = pb.thr;
   pa.flip2 = pb.flip;

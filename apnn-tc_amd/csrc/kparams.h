@@ -54,7 +54,7 @@ struct KParams {
   int pair_tiles;            // 0: single problem
   const uint32_t *B2;
   int KW2, S2, pad2;
-  uint32_t magicS2;
+  uint32_t magicS2, magicS16_2;
   long long planeB2;
   const int32_t *thr2;
   const uint8_t *flip2;

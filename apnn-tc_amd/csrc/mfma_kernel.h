@@ -844,6 +844,7 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
     p.S = pk.S2;
     p.pad = pk.pad2;
     p.magicS = pk.magicS2;
+    p.magicS16 = pk.magicS16_2;
     p.planeB = pk.planeB2;
     p.thr = pk.thr2;
     p.flip = pk.flip2;

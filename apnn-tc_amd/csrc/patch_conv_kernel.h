@@ -88,15 +88,42 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
 #pragma unroll
   for (int x = 0; x < FA; ++x) prow[x] = row_base(min((wa * FA + x) * 32 + li, last_row - a0)) - q_lo;
 
-  // patch pixels this thread stages: global word offset of the pixel (channel word 0), or -1 for
+  // Global loads go through one buffer descriptor per operand plane (base, size in bytes; the host launches
+  // this kernel only for planes below 4 GiB): a load whose offset lies past the descriptor's size returns
+  // zeros, so padding pixels, rows past the end and the unused tail of a task batch are the same instruction
+  // with the offset 0xffffffff instead of a branch around the load.
+  constexpr uint32_t kOff = 0xffffffffu;
+  __amdgpu_buffer_rsrc_t rsrcA[PA], rsrcB[PB];
+#pragma unroll
+  for (int pl = 0; pl < PA; ++pl)
+    rsrcA[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.A + pl * p.planeA), 0,
+                                                  (int)(uint32_t)(p.planeA * 4), 0x00020000);
+#pragma unroll
+  for (int pl = 0; pl < PB; ++pl)
+    rsrcB[pl] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.B + pl * p.planeB), 0,
+                                                  (int)(uint32_t)(p.planeB * 4), 0x00020000);
+  // word pair at byte offset boff (kOff: zeros); without 64-bit loads (odd number of channel words) the
+  // second word of the last pair does not exist
+  auto load_pair = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t boff, auto pair_c, bool second, uint32_t &w0,
+                       uint32_t &w1) {
+    if constexpr (decltype(pair_c)::value) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)boff, 0, 0);
+      w0 = v[0], w1 = v[1];
+    } else {
+      w0 = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)boff, 0, 0);
+      w1 = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(second && boff != kOff ? boff + 4 : kOff), 0, 0);
+    }
+  };
+
+  // patch pixels this thread stages: byte offset of the pixel (channel word 0) in a plane, or kOff for
   // padding / beyond the range
-  long long poff[PATCH_NPT];
+  uint32_t poff[PATCH_NPT];
   const int pad_v = (p.PHs - p.Hs) >> 1;
   const int yp0 = gy0 * gst, xp0 = gx0 * gst;
 #pragma unroll
   for (int j = 0; j < PATCH_NPT; ++j) {
     const int q = tid + j * NT;
-    poff[j] = -1;
+    poff[j] = kOff;
     if (q < npp) {
       int xp = xp0 + q;
       const int cy = (int)fast_div((uint32_t)xp, (uint32_t)p.PWs, p.magicPW);
@@ -107,7 +134,7 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
       const int img = b0i + ci;
       const int iy = yp - pad_v, ix = xp - pad_v;
       if (img < p.batch && iy >= 0 && iy < p.Hs && ix >= 0 && ix < p.Ws)
-        poff[j] = (((long long)img * p.Hs + iy) * p.Ws + ix) * p.C32;
+        poff[j] = ((((uint32_t)img * (uint32_t)p.Hs + (uint32_t)iy) * (uint32_t)p.Ws + (uint32_t)ix) * (uint32_t)p.C32) << 2;
     }
   }
 
@@ -133,50 +160,35 @@ __global__ __launch_bounds__(256, OCC) void apnn_patch_conv_kernel(const KParams
     // ---- global loads of the chunk: patch pixels, then the first batch of filter tasks; all are in
     // flight before the first one is consumed ----------------------------------------------------
     uint32_t pw0[PATCH_NPT][PA], pw1[PATCH_NPT][PA];
+    const bool second = cw + 1 < p.C32;
+    // (one branch on the load width around each batch of loads, not one per load)
+    auto patch_load = [&](auto pair_c) {
 #pragma unroll
-    for (int j = 0; j < PATCH_NPT; ++j) {
-      const bool in = poff[j] >= 0;
+      for (int j = 0; j < PATCH_NPT; ++j) {
+        const uint32_t boff = poff[j] != kOff ? poff[j] + ((uint32_t)cw << 2) : kOff;
 #pragma unroll
-      for (int pl = 0; pl < PA; ++pl) {
-        pw0[j][pl] = pw1[j][pl] = 0;
-        if (in) {
-          const uint32_t *src = p.A + pl * p.planeA + poff[j] + cw;
-          if (pair_ok) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(src);
-            pw0[j][pl] = v.x;
-            pw1[j][pl] = v.y;
-          } else {
-            pw0[j][pl] = src[0];
-            if (cw + 1 < p.C32) pw1[j][pl] = src[1];
-          }
-        }
+        for (int pl = 0; pl < PA; ++pl) load_pair(rsrcA[pl], boff, pair_c, second, pw0[j][pl], pw1[j][pl]);
       }
-    }
+    };
+    if (pair_ok) patch_load(std::true_type{}); else patch_load(std::false_type{});
     constexpr int FT = 4;  // filter tasks (tap, column) per thread and batch
     const int ntask = taps * TB;
     uint32_t fw0[FT][PB], fw1[FT][PB];
-    auto filter_load = [&](int first) {
+    auto filter_load_w = [&](int first, auto pair_c) {
 #pragma unroll
       for (int j = 0; j < FT; ++j) {
         const int t = first + tid + j * NT;
         const int tap = t / TB, col = t % TB;
         const int gcol = b0 + col;
+        const uint32_t boff = t < ntask && gcol < p.rowsB
+                                  ? (((uint32_t)gcol * (uint32_t)taps + (uint32_t)tap) * (uint32_t)p.C32 + (uint32_t)cw) << 2
+                                  : kOff;
 #pragma unroll
-        for (int pl = 0; pl < PB; ++pl) {
-          fw0[j][pl] = fw1[j][pl] = 0;
-          if (t < ntask && gcol < p.rowsB) {
-            const uint32_t *src = p.B + pl * p.planeB + ((long long)gcol * taps + tap) * p.C32 + cw;
-            if (pair_ok) {
-              const uint2 v = *reinterpret_cast<const uint2 *>(src);
-              fw0[j][pl] = v.x;
-              fw1[j][pl] = v.y;
-            } else {
-              fw0[j][pl] = src[0];
-              if (cw + 1 < p.C32) fw1[j][pl] = src[1];
-            }
-          }
-        }
+        for (int pl = 0; pl < PB; ++pl) load_pair(rsrcB[pl], boff, pair_c, second, fw0[j][pl], fw1[j][pl]);
       }
+    };
+    auto filter_load = [&](int first) {
+      if (pair_ok) filter_load_w(first, std::true_type{}); else filter_load_w(first, std::false_type{});
     };
     auto filter_store = [&](int first) {
 #pragma unroll

@@ -364,12 +364,10 @@ def main():
                        R=3, S=3, stride=1, pad=1, halo=1, wb=w_, xb=a_, weight_mode=A.WEIGHT_UNSIGNED, epi=E,
                        path=cur["path"])
         ev, wall = ctypes.c_float(), ctypes.c_double()
-        if batch == 1:
-            A.check(benchlib.apnn_bench_conv_graph(ctypes.byref(d), warmup, iters, GRAPH_BATCH, ctypes.byref(ev),
-                                                   ctypes.byref(wall)), "apnn_bench_conv_graph")
-        else:
-            A.check(benchlib.apnn_bench_conv(ctypes.byref(d), warmup, iters, stream, ctypes.byref(ev),
-                                             ctypes.byref(wall)), "apnn_bench_conv")
+        # graph replay at both batch sizes: a plain launch loop issues a kernel every 3-5 us at best, which
+        # would hide every batch-16 row that runs faster than that
+        A.check(benchlib.apnn_bench_conv_graph(ctypes.byref(d), warmup, iters, min(GRAPH_BATCH, iters), ctypes.byref(ev),
+                                               ctypes.byref(wall)), "apnn_bench_conv_graph")
         torch.cuda.synchronize()
         rows = batch * H * Wd
         if fused:
@@ -442,7 +440,7 @@ def main():
                     # sizes, for all four precisions
                     for C in (128, 256, 384, 512, 640, 768, 896, 1024):
                         for fused in (False, True):
-                            t = time_conv(batch, C, w_, a_, fused, 200 if batch == 1 else 10, 1000 if batch == 1 else 50)
+                            t = time_conv(batch, C, w_, a_, fused, 200 if batch == 1 else 20, 1000 if batch == 1 else 100)
                             t["shape"] = "w%da%d 3x3 16x16 b%d Cin=Cout=%d %s" % (
                                 w_, a_, batch, C, "bn-quantize packed out" if fused else "int32 out")
                             convs.append(t)
@@ -507,7 +505,7 @@ def main():
         else:
             bt, Cc = int(f[2][1:]), int(f[3][1:])
             Hm = int(f[5][1:]) if len(f) > 5 else 16
-            t = time_conv(bt, Cc, w_, a_, f[4] == "fused", 200 if bt == 1 else 10, 1000 if bt == 1 else 50, H=Hm)
+            t = time_conv(bt, Cc, w_, a_, f[4] == "fused", 200 if bt == 1 else 20, 1000 if bt == 1 else 100, H=Hm)
             t.update(shape=spec, path=args.path)
             extra.setdefault("requested", []).append(t)
     if "crossover" in want:

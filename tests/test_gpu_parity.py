@@ -1101,3 +1101,39 @@ def test_conv_pair_residual_block_entry(G, batch, H, C, cout, wb, xb):
     bad = desc(dW1, o1, 1, 0, dT1)
     bad.stride = 1
     assert A.lib().apnn_conv_pair(ctypes.byref(da), ctypes.byref(bad), None) == A.EINVAL
+
+
+@pytest.mark.parametrize("batch,H,C,cout,stride", [(4, 14, 256, 128, 1), (3, 20, 128, 256, 2), (16, 14, 64, 64, 1)])
+def test_conv_pair_two_filter_sizes(G, batch, H, C, cout, stride):
+    """apnn_conv_pair with two filters that both span several taps and differ in width (5x5 pad 2 and 3x3
+    pad 1 produce the same output grid): the second problem decodes its taps with its own filter width."""
+    rng = np.random.default_rng(8100 + batch + H)
+    wb, xb = 1, 2
+    X = O.random_planes(rng, xb, batch * H * H, C // 32)
+    W5 = O.random_planes(rng, wb, cout * 25, C // 32)
+    W3 = O.random_planes(rng, wb, cout * 9, C // 32)
+    k5 = dict(batch=batch, H=H, W=H, cout=cout, R=5, S=5, stride=stride, pad=2, halo=0, wb=wb, xb=xb)
+    k3 = dict(batch=batch, H=H, W=H, cout=cout, R=3, S=3, stride=stride, pad=1, halo=0, wb=wb, xb=xb)
+    acc5 = O.conv(W5, X, cwords=C // 32, sym_w=1, nthreads=8, **k5).reshape(-1, cout)
+    acc3 = O.conv(W3, X, cwords=C // 32, sym_w=1, nthreads=8, **k3).reshape(-1, cout)
+    rows = acc5.shape[0]
+    assert acc3.shape[0] == rows
+    thr5 = np.sort(rng.integers(int(acc5.min()), int(acc5.max()) + 1, size=(cout, 3)), axis=1).astype(np.int32)
+    thr3 = np.sort(rng.integers(int(acc3.min()), int(acc3.max()) + 1, size=(cout, 3)), axis=1).astype(np.int32)
+    dX, dW5, dW3, dT5, dT3 = G.to_dev(X), G.to_dev(W5), G.to_dev(W3), G.to_dev(thr5), G.to_dev(thr3)
+    words = xb * rows * cout // 32
+    A = G.A
+    def desc(Wd_, out, R, pad, thr):
+        return A.ConvDesc(W=Wd_.data_ptr(), X=dX.data_ptr(), O=out.data_ptr(), batch=batch, H=H, Wd=H, cin_pad=C,
+                          COUT=cout, R=R, S=R, stride=stride, pad=pad, halo=0, wb=wb, xb=xb,
+                          weight_mode=A.WEIGHT_SYMMETRIC, epi=G.epilogue(mode=A.EPI_BN, out_bits=xb, thr=thr),
+                          path=A.PATH_AUTO)
+    e5 = O.lowbits_pack(O.bn_quantize(acc5, None, thr5, None, xb), rows, cout, xb)
+    e3 = O.lowbits_pack(O.bn_quantize(acc3, None, thr3, None, xb), rows, cout, xb)
+    for first_is_5 in (True, False):
+        o5, o3 = G.dev_empty_i32(words, fill=-7), G.dev_empty_i32(words, fill=-7)
+        d5, d3 = desc(dW5, o5, 5, 2, dT5), desc(dW3, o3, 3, 1, dT3)
+        da, db = (d5, d3) if first_is_5 else (d3, d5)
+        A.check(A.lib().apnn_conv_pair(ctypes.byref(da), ctypes.byref(db), None), "apnn_conv_pair")
+        assert np.array_equal(G.to_host(o5, np.uint32).reshape(e5.shape), e5), first_is_5
+        assert np.array_equal(G.to_host(o3, np.uint32).reshape(e3.shape), e3), first_is_5
