@@ -366,7 +366,7 @@ int from_hip(hipError_t e) { return e == hipErrorNotSupported ? APNN_EUNSUPPORTE
 // is the one done four times per k-step; then 128x128, 64x64 (128x64 for <= 64 output channels) while every
 // compute unit still gets a work-group; when even 64x64 tiles leave most of the chip idle and the
 // reduction is long, the 32-row tiles whose four waves split K.
-int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3) {
+int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, int planes = 3, int planesW = 1) {
   const bool wide = planes > 5 || planes == 2;  // the reduced tile set (see mfma_tile_enabled)
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -399,22 +399,30 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
   // About one 128x128 tile per compute unit over a long reduction (16x16 maps at batch 16 with 1024 channels,
   // 14x14x256 at batch 64, 2048^2 outputs): plain 128x128 work-groups would leave one wave per SIMD, so two
   // wave groups share each tile's k-steps.  Measured 11-18 % ahead of the best other tile there; with fewer
-  // tiles than that the idle compute units cost more than the split-K tiles' extra operand traffic
-  // (3/4 of the units busy against the 32x32 / 32x64 split-K tiles, 9/10 against 32x128).
+  // tiles than that the idle compute units cost more than the split-K tiles' extra operand traffic.  How
+  // many units may idle depends on what the 32x64 split-K tile costs instead: with one weight plane and
+  // either many channel blocks or three and more activation planes it stays ahead until 9/10 of the units
+  // have a tile (16x16 maps with 640..896 channels, 14x14x256 at batch 64 for w1a3 / w1a4); with two weight
+  // planes, whose expansion the small tiles repeat per 64 channels, and for the GEMM entry points 3/4 suffice
+  // (w2a2 on 16x16 maps: 17 % ahead at 768 channels, 34 % at 896).
   if ((!conv || vw == 4) && planes > 2 && KW >= 64 && fill(1) >= 0.8) {
     const long long nt1 = ntiles(1);
-    const bool wide_split_ok = conv && rowsB >= 512;  // the 32x128 split-K tile applies
-    if (2 * nt1 < 3 * cus && (wide_split_ok ? 10 * nt1 >= 9 * cus : 4 * nt1 >= 3 * cus)) return apnn::MT_128x128_G2;
+    const bool strict = conv && planesW == 1 && (rowsB >= 512 || planes >= 4);
+    if (2 * nt1 < 3 * cus && (strict ? 10 * nt1 >= 9 * cus : 4 * nt1 >= 3 * cus)) return apnn::MT_128x128_G2;
   }
   // Few outputs over a long reduction (batch-1 / batch-8 layers, 7x7 maps): the split-K tiles give
   // every 32x32 (32x64) block a work-group of its own and the four waves share K.  Measured
   // cross-overs on ResNet18 / 16x16 benchmark shapes.
   if (conv) {
     const long long nb32 = ntiles(4);
-    // Long reduction, at least 512 output channels and enough 32x128 tiles for 1.5 work-groups per
-    // compute unit (7x7x512 maps at batch 64, 16x16x512..1024 at batch 16): one activation expansion feeds
-    // four blocks, 11-16 % faster than 32x64 / 128x64 there; with 256 channels or fewer tiles it loses
-    if (vw == 4 && KW >= 64 && rowsB >= 512 && 2 * ntiles(8) >= 3 * cus && nb32 <= 4096) return 8;
+    // 32x128 split-K tile: one activation expansion feeds four channel blocks.  It pays with four
+    // activation planes over a long reduction while all its work-groups are resident at once (1.5 to 2 per
+    // compute unit: 7x7x512 maps at batch 64, 16x16x512 at batch 16; 4-5 % ahead of 32x64).  With fewer
+    // activation planes 32x64 is level or ahead, and a grid of 2.5 to 3.5 work-groups per unit pays for the
+    // larger tile's longer last round (16x16 maps with 640..896 channels: 32x64 5-20 % ahead).
+    if (vw == 4 && planes >= 5 && planesW == 1 && KW >= 128 && rowsB >= 512 && 2 * ntiles(8) >= 3 * cus &&
+        ntiles(8) <= 2 * cus)
+      return 8;
     // 32x32 blocks, one work-group each: with three planes in all while every compute unit gets at most one
     // (from 296 blocks the 32x64 tile, whose wave expands an activation block once for two channel blocks,
     // is 5-9 % ahead with quantized output and level with int32 output); with four or more planes up to 2.5
@@ -422,7 +430,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
     // ahead up to 592 blocks, 32x64 takes over at 784).  Measured on 14x14x256 maps at batch 4..16.
     if (KW >= 32 && nb32 <= (planes <= 3 ? 256 : 640)) return 4;
     if (KW >= 32 && nb32 <= 640) return 5;
-    if (KW >= 64 && nb32 <= 3200) return 5;
+    if (KW >= 64 && nb32 <= 14 * cus) return 5;  // up to 3584 blocks: 16x16 maps at batch 16, 896 channels
   }
   if (rowsB <= 64 && ntiles(3) >= cus) return 3;
   if (rowsB > 64) {
@@ -448,7 +456,7 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
 
 int pick_mfma_tile(int tile_pin, const KParams &p, bool conv, int vw, bool i8, int *tile) {
   if (tile_pin == 0) {
-    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB);
+    *tile = choose_mfma_tile(p.rowsA, p.rowsB, p.KW, conv, vw, i8, p.planesA + p.planesB, conv ? p.planesB : p.planesA);
     return APNN_OK;
   }
   if (tile_pin - 1 >= apnn::kMfmaTileCount) return APNN_EINVAL;
@@ -766,7 +774,7 @@ int run_conv_pair(const apnn_conv_desc *a, const apnn_conv_desc *b, hipStream_t 
     return run_conv(b, stream);
   }
   // tile for the larger of the two problems, evaluated for twice the number of work-groups
-  int tile = choose_mfma_tile(2 * pa.rowsA, pa.rowsB, pa.KW, true, vwa, false);
+  int tile = choose_mfma_tile(2 * pa.rowsA, pa.rowsB, pa.KW, true, vwa, false, a->xb + a->wb, a->wb);
   pa.pair_tiles = 1;  // flag; the launcher fills in the tile count
   pa.B2 = pb.B;
   pa.KW2 = pb.KW;

@@ -45,6 +45,9 @@ struct KParams {
   // tap / S with magicS16 = ceil(65536 / S); stored width, C32 and KW below 2^24.
   // c32_shift: log2(C32) when C32 is a power of two, else -1.
   int addr32, c32_shift;
+  // Matrix-core kernels, set by the launcher: 0, or the height (in tile rows) of the bands in which the
+  // work-groups of one XCD walk the tile grid (see apnn_mfma_kernel's tile decode).
+  int xcd_rows;
   uint32_t magicS16;
 
   // Paired launch (matrix-core convolution kernels only): work-groups pair_tiles .. 2*pair_tiles-1

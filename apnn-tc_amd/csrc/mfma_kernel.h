@@ -881,9 +881,26 @@ __global__ __launch_bounds__(256 * KSX, OCC) void apnn_mfma_kernel(const KParams
   const int wv = KSX > 1 ? wave & 3 : wave; // wave within its group
   const int wa = KS > 1 ? 0 : wv / WB, wb = KS > 1 ? 0 : wv % WB;
 
+  // Work-group index -> tile.  Consecutive indices land on different XCDs (round-robin over the eight), each
+  // with an L2 of its own.  In row-major order the work-groups of one XCD would therefore take every eighth
+  // tile of every row band and each L2 would fetch all of one operand.  With xcd_rows set (large grids) the
+  // index is regrouped into one contiguous range of tiles per XCD, and a range walks the grid in bands of
+  // xcd_rows tile rows, column by column: the work-groups resident on an XCD at one time share a few row
+  // blocks and a few column blocks in that XCD's L2.
   const int tilesB = (p.rowsB + TB - 1) / TB;
-  const int a0 = (bid / tilesB) * TA;
-  const int b0 = (bid % tilesB) * TB;
+  int trow = bid / tilesB, tcol = bid % tilesB;
+  if (p.xcd_rows > 0) {
+    const int tilesA = (p.rowsA + TA - 1) / TA;
+    const int per_xcd = (tilesA * tilesB) >> 3;  // the launcher checked that the grid is a multiple of 8
+    const int lin = (bid & 7) * per_xcd + (bid >> 3);
+    const int per_band = p.xcd_rows * tilesB;
+    const int band = lin / per_band, w = lin - band * per_band;
+    const int rows_in_band = min(p.xcd_rows, tilesA - band * p.xcd_rows);
+    tcol = w / rows_in_band;
+    trow = band * p.xcd_rows + (w - tcol * rows_in_band);
+  }
+  const int a0 = trow * TA;
+  const int b0 = tcol * TB;
 
   // output pixel (row of A) -> image index and the input coordinates of its filter tap (0, 0)
   auto pixel_origin = [&](int pix, int &b, int &y0, int &x0) {
@@ -1451,6 +1468,8 @@ constexpr size_t mfma_smem_bytes(int core, int PA, int PB, int FA, int FB, int W
 }
 
 // OCC_WANTED work-groups per compute unit, or as many as the LDS budget (160 KiB) allows
+constexpr long long kXcdOrderMinTiles = 256;
+
 template <int CORE, int PA, int PB, int FA, int FB, int WA, int WB, int VW, bool CONV, int OCC_WANTED, int KSX = 1>
 inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   constexpr int TA = WA * FA * 32, TB = WB * FB * 32;
@@ -1471,6 +1490,10 @@ inline hipError_t launch_mfma(const KParams &p, hipStream_t stream) {
   const long long tiles = (long long)((p.rowsA + TA - 1) / TA) * ((p.rowsB + TB - 1) / TB);
   KParams q = p;
   if (p.pair_tiles != 0) q.pair_tiles = (int)tiles;  // the host only flags a pair; the tile count is known here
+  // XCD-aware tile order for grids of at least one work-group per compute unit (smaller grids are over
+  // before the L2s matter, and the regrouping costs every work-group two scalar divisions)
+  const long long tilesB = (p.rowsB + TB - 1) / TB;
+  q.xcd_rows = (p.pair_tiles == 0 && tiles % 8 == 0 && tiles >= kXcdOrderMinTiles && tilesB >= 2) ? 8 : 0;
   hipLaunchKernelGGL(kern, dim3((unsigned)(q.pair_tiles != 0 ? 2 * tiles : tiles)), dim3(256 * KSX), smem_bytes, stream,
                      q);
   return hipGetLastError();

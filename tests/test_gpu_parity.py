@@ -1103,6 +1103,28 @@ def test_conv_pair_residual_block_entry(G, batch, H, C, cout, wb, xb):
     assert A.lib().apnn_conv_pair(ctypes.byref(da), ctypes.byref(bad), None) == A.EINVAL
 
 
+@pytest.mark.parametrize("M,N,path,tile", [
+    (1500, 3022, 2, 1),    # 12 x 24 tiles of 128x128: one full band of eight tile rows and a band of four
+    (1100, 4000, 2, 1),    # 9 x 32: a band of eight and a band of one
+    (1100, 4000, 3, 1),    # the same grid on the int8 core
+    (2048, 2048, 2, 9),    # 16 x 16 on the two-wave-group tile
+    (520, 4090, 2, 2),     # 9 x 64 tiles of 64x64
+    (3000, 1400, 2, 3),    # 24 x 22 tiles of 128x64
+    (2530, 4096, 2, 6)])   # 10 x 32 tiles of 256x128: a band of eight and a band of two
+def test_gemm_grids_walked_in_xcd_order(G, M, N, path, tile):
+    """Grids of at least 256 tiles whose size is a multiple of eight are walked in per-XCD ranges, in
+    bands of eight tile rows (the work-group index is regrouped inside the kernel): every tile, ragged
+    edges included, is computed exactly once -- the whole output equals the oracle's, and nothing is
+    written outside it (guard bytes)."""
+    K, wb, xb = 256, 1, 2
+    rng = np.random.default_rng(8200 + M + N + tile)
+    W = O.random_planes(rng, wb, M, K // 32)
+    X = O.random_planes(rng, xb, N, K // 32)
+    ref = O.gemm(W, X, M, N, K, wb, xb, sym_w=1, nthreads=8)
+    got = G.run_gemm(W, X, M, N, K, wb, xb, sym=1, path=path, tile=tile).reshape(M, N)
+    assert np.array_equal(got, ref)
+
+
 @pytest.mark.parametrize("batch,H,C,cout,stride", [(4, 14, 256, 128, 1), (3, 20, 128, 256, 2), (16, 14, 64, 64, 1)])
 def test_conv_pair_two_filter_sizes(G, batch, H, C, cout, stride):
     """apnn_conv_pair with two filters that both span several taps and differ in width (5x5 pad 2 and 3x3
