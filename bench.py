@@ -133,6 +133,71 @@ def crossover_table(A, G, O, benchlib, stream):
     return out
 
 
+def crossover_sweep(A, G, O, benchlib):
+    """The library's own choice against every FP4 matrix-core tile that is built, over the whole 16x16
+    convolution sweep (four precisions x batch 1 / 16 x eight channel counts x int32 / quantized output) and
+    ten GEMM sizes per precision: the measurement behind the per-precision tile rules of the dispatcher.
+    Every candidate and AUTO are replayed from HIP graphs in the same process; `ratio` = AUTO / fastest tile."""
+    import numpy as np
+    import torch
+    KN = {A.KERNEL_VALU_TILE: "valu", A.KERNEL_VALU_DIRECT: "valu-direct", A.KERNEL_MFMA_FP4: "fp4",
+          A.KERNEL_MFMA_I8: "i8", A.KERNEL_PATCH_FP4: "patch", A.KERNEL_MFMA_FP4_XS: "xs"}
+    rng = np.random.default_rng(0x5EED0005)
+    L = A.lib()
+
+    def run(fn, desc, n):
+        ev, wall = ctypes.c_float(), ctypes.c_double()
+        rc = fn(ctypes.byref(desc), max(20, n // 5), n, min(GRAPH_BATCH, n), ctypes.byref(ev), ctypes.byref(wall))
+        torch.cuda.synchronize()
+        return None if rc != 0 else ev.value / n * 1e3
+
+    def sweep(name, desc, plan_fn, fn, n, tiles):
+        plan = A.Plan()
+        desc.path = A.PATH_AUTO
+        assert plan_fn(ctypes.byref(desc), ctypes.byref(plan)) == 0
+        times = {}
+        for t in tiles:
+            desc.path = A.PATH_MFMA | ((t + 1) << 8)
+            if plan_fn(ctypes.byref(desc), ctypes.byref(A.Plan())) != 0:
+                continue
+            v = run(fn, desc, n)
+            if v is not None:
+                times[t] = round(v, 2)
+        desc.path = A.PATH_AUTO
+        ta = run(fn, desc, n)
+        best = min(times, key=times.get)
+        return {"shape": name, "auto": "%s/%d" % (KN[plan.kernel], plan.tile), "auto_us": round(ta, 2), "best_tile": best,
+                "best_us": times[best], "ratio": round(ta / times[best], 3), "tiles_us": times}
+
+    out = []
+    for (wb, xb) in [(1, 2), (1, 3), (1, 4), (2, 2)]:
+        for batch in (1, 16):
+            for C in (128, 256, 384, 512, 640, 768, 896, 1024):
+                for fused in (False, True):
+                    H = 16
+                    rows = batch * H * H
+                    X = G.to_dev(O.random_planes(rng, xb, rows, C // 32))
+                    Wt = G.to_dev(O.random_planes(rng, wb, C * 9, C // 32))
+                    thr = G.to_dev(np.sort(rng.integers(-200, 200, size=(C, 2 ** xb - 1)), axis=1).astype(np.int32))
+                    outp = G.dev_empty_i32(max(xb * rows * C // 32, rows * C))
+                    E = G.epilogue(mode=A.EPI_BN, out_bits=xb, thr=thr) if fused else G.epilogue()
+                    d = A.ConvDesc(W=Wt.data_ptr(), X=X.data_ptr(), O=outp.data_ptr(), batch=batch, H=H, Wd=H, cin_pad=C,
+                                   COUT=C, R=3, S=3, stride=1, pad=1, halo=0, wb=wb, xb=xb,
+                                   weight_mode=A.WEIGHT_UNSIGNED, epi=E)
+                    out.append(sweep("conv w%da%d 16x16 b%d C=%d %s" % (wb, xb, batch, C, "bn-packed" if fused else "int32"),
+                                     d, L.apnn_conv_plan, benchlib.apnn_bench_conv_graph,
+                                     1000 if rows * C * C < 3e9 else 200, (1, 2, 3, 4, 5, 7, 8, 9)))
+        for (M, N, K) in [(512, 512, 1024), (1024, 1024, 1024), (1024, 1024, 4096), (2048, 2048, 2048), (1024, 4096, 2048),
+                          (4096, 1024, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (2048, 8192, 4096), (6144, 6144, 6144)]:
+            W = G.to_dev(O.random_planes(rng, wb, M, K // 32))
+            X = G.to_dev(O.random_planes(rng, xb, N, K // 32))
+            D = G.dev_empty_i32(M * N)
+            d = A.GemmDesc(W=W.data_ptr(), X=X.data_ptr(), D=D.data_ptr(), M=M, N=N, K=K, wb=wb, xb=xb)
+            out.append(sweep("gemm w%da%d %dx%dx%d" % (wb, xb, M, N, K), d, L.apnn_gemm_plan, benchlib.apnn_bench_gemm_graph,
+                             500 if M * N * K < 2e10 else 40, (1, 2, 3, 4, 5, 6, 9)))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,7 +209,9 @@ def main():
                     help="comma list of secondary workloads to run after the headline: all, none, gemm_sweep, "
                          "gemm_large, gemm8192 (w1a2 only), conv, nets, resnet18_b8, resnet18_b64, alexnet_b8, "
                          "alexnet_b64, vgg_b8, vgg_b64; crossover (not part of all): every kernel path / tile "
-                         "pinned in turn on the shapes where the library's choice changes")
+                         "pinned in turn on the shapes where the library's choice changes; crossover_sweep (not part "
+                         "of all): AUTO against every FP4 matrix-core tile over the whole convolution sweep and ten "
+                         "GEMM sizes, all four precisions")
     ap.add_argument("--path", default="auto")
     ap.add_argument("--shape", action="append", default=[],
                     help="extra workload on --path (repeatable; used by the profile commands): "
@@ -510,6 +577,8 @@ def main():
             extra.setdefault("requested", []).append(t)
     if "crossover" in want:
         extra["crossover"] = crossover_table(A, G, O, benchlib, stream)
+    if "crossover_sweep" in want:
+        extra["crossover_sweep"] = crossover_sweep(A, G, O, benchlib)
     result["extra"] = extra
 
     # ---- CPU baseline: the scalar oracle on the same inputs, host cores ---------------------------
