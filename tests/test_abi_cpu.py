@@ -284,6 +284,25 @@ def test_plan_reports_the_dispatchers_choices():
     rc, plan = _plan_conv(batch=64, H=56, Wd=56, cin_pad=64, COUT=64, R=3, S=3, stride=1, pad=1, halo=0, wb=1, xb=2,
                           path=A.PATH_AUTO)
     assert rc == 0 and plan.kernel == A.KERNEL_PATCH_FP4 and plan.patch_pixels > 0
+    # per-precision tile rules on the 16x16 batch-16 sweep (tile shape and split-K factor as measured fastest)
+    def conv16(C, wb, xb):
+        rc, pl = _plan_conv(batch=16, H=16, Wd=16, cin_pad=C, COUT=C, R=3, S=3, stride=1, pad=1, halo=1, wb=wb, xb=xb,
+                            path=A.PATH_AUTO)
+        assert rc == 0 and pl.kernel == A.KERNEL_MFMA_FP4
+        return (pl.tile_rows, pl.tile_cols, pl.split_k)
+    assert conv16(1024, 1, 2) == (128, 128, 2)      # one 128x128 tile per compute unit: two wave groups
+    assert conv16(896, 1, 2) == (32, 64, 4)         # 7/8 of the units would get a tile: 32x64 split-K is ahead
+    assert conv16(896, 2, 2) == (128, 128, 2)       # two weight planes: the two-wave-group tile from 3/4
+    assert conv16(640, 2, 2) == (32, 64, 4)
+    assert conv16(512, 1, 4) == (32, 128, 4)        # four activation planes, all work-groups resident at once
+    assert conv16(512, 1, 2) == (32, 64, 4)
+    assert conv16(128, 1, 4) == (32, 32, 4)         # 512 blocks of 32x32 with five planes in all
+    assert conv16(128, 1, 2) == (32, 64, 4)
+    # the kernel that expands operands while staging is reachable by pinning only
+    rc, plan = _plan_gemm(M=8192, N=8192, K=8192, wb=1, xb=4, path=A.PATH_AUTO)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4 and plan.path == A.PATH_MFMA
+    rc, plan = _plan_gemm(M=8192, N=8192, K=8192, wb=1, xb=4, path=A.PATH_MFMA_XS)
+    assert rc == 0 and plan.kernel == A.KERNEL_MFMA_FP4_XS
     assert A.lib().apnn_gemm_plan(None, ctypes.byref(A.Plan())) == A.ENULL
     g = A.GemmDesc(W=0x1000, X=0x1000, D=0x1000, M=64, N=64, K=128, wb=1, xb=2)
     assert A.lib().apnn_gemm_plan(ctypes.byref(g), None) == A.ENULL
