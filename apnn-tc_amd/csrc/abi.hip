@@ -325,7 +325,8 @@ int patch_pixels(const KParams &p, int R, int rows) {
 // 1024 pixels) and the filter block of all taps must fit in LDS twice per compute unit.  When the
 // library chooses (`automatic`) the kernel is taken only where it measures faster than the
 // implicit-GEMM kernel: at most 64 output channels over at most 64 input channels (one channel
-// chunk, e.g. the first stage of ResNet18) with enough 128x64 tiles to occupy the chip.
+// chunk, e.g. the first stage of ResNet18) with enough 128x64 tiles to occupy the chip, and layers whose
+// channel words are odd in number.
 int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
   int cus = device_cus();
   if (cus <= 0) cus = 256;
@@ -344,7 +345,12 @@ int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
   if (automatic) {
     if (tile_pin != 0) return -1;  // a pinned tile names a tile of the implicit-GEMM families
     const int t = 3;               // 128 x 64
-    return (p.rowsB <= 64 && p.C32 <= 2 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus) ? t : -1;
+    if (p.rowsB <= 64 && p.C32 <= 2 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus) return t;
+    // An odd number of channel words (96 channels: the second layer of the VGG variant) leaves the
+    // implicit-GEMM kernel with 32-bit loads and its two smallest tiles; this kernel reads pixels, not
+    // k-chunks, and is 22-34 % ahead there (56x56x96 -> 256 at batch 8 / 64).
+    if ((p.C32 & 1) && p.C32 >= 3 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus) return t;
+    return -1;
   }
   if (tile_pin != 0) {
     const int t = tile_pin - 1;
@@ -400,14 +406,14 @@ int choose_mfma_tile(int rowsA, int rowsB, int KW, bool conv, int vw, bool i8, i
   // 14x14x256 at batch 64, 2048^2 outputs): plain 128x128 work-groups would leave one wave per SIMD, so two
   // wave groups share each tile's k-steps.  Measured 11-18 % ahead of the best other tile there; with fewer
   // tiles than that the idle compute units cost more than the split-K tiles' extra operand traffic.  How
-  // many units may idle depends on what the 32x64 split-K tile costs instead: with one weight plane and
-  // either many channel blocks or three and more activation planes it stays ahead until 9/10 of the units
-  // have a tile (16x16 maps with 640..896 channels, 14x14x256 at batch 64 for w1a3 / w1a4); with two weight
+  // many units may idle depends on what the 32x64 split-K tile costs instead: in convolutions with one
+  // weight plane it stays ahead until 9/10 of the units have a tile (16x16 maps with 640..896 channels;
+  // 14x14x256 at batch 64: 5 % ahead for w1a2 with quantized output, 17 % for w1a3 / w1a4); with two weight
   // planes, whose expansion the small tiles repeat per 64 channels, and for the GEMM entry points 3/4 suffice
   // (w2a2 on 16x16 maps: 17 % ahead at 768 channels, 34 % at 896).
   if ((!conv || vw == 4) && planes > 2 && KW >= 64 && fill(1) >= 0.8) {
     const long long nt1 = ntiles(1);
-    const bool strict = conv && planesW == 1 && (rowsB >= 512 || planes >= 4);
+    const bool strict = conv && planesW == 1;
     if (2 * nt1 < 3 * cus && (strict ? 10 * nt1 >= 9 * cus : 4 * nt1 >= 3 * cus)) return apnn::MT_128x128_G2;
   }
   // Few outputs over a long reduction (batch-1 / batch-8 layers, 7x7 maps): the split-K tiles give
