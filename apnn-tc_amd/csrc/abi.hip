@@ -349,7 +349,9 @@ int choose_patch_tile(const KParams &p, int R, int tile_pin, bool automatic) {
     // An odd number of channel words (96 channels: the second layer of the VGG variant) leaves the
     // implicit-GEMM kernel with 32-bit loads and its two smallest tiles; this kernel reads pixels, not
     // k-chunks, and is 22-34 % ahead there (56x56x96 -> 256 at batch 8 / 64).
-    if ((p.C32 & 1) && p.C32 >= 3 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus) return t;
+    // (256x64 tiles while 128x64 would give fewer than four work-groups per compute unit: 9 % ahead at batch 8)
+    if ((p.C32 & 1) && p.C32 >= 3 && taps > 1 && fits(t) && ntiles(t) >= 2 * cus)
+      return (ntiles(t) < 4 * cus && fits(1)) ? 1 : t;
     return -1;
   }
   if (tile_pin != 0) {
