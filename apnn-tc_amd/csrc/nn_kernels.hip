@@ -631,32 +631,62 @@ __global__ __launch_bounds__(64 * NWAV, NWAV == 8 ? 4 : 1) void conv_i8_rows_ker
 // ---- max-pool directly on bit-planes ----------------------------------------------------------------
 // in: [bits][B*H*W][cw] -> out: [bits][B*Ho*Wo][cw]; the maximum of two multi-bit codes is computed for
 // 32 channels at once with bitwise logic (compare from the top plane down).
-// NB: planes held in registers (2 for the usual one- and two-bit codes, else 8).
-template <int NB>
+// NB: planes held in registers (2 for the usual one- and two-bit codes, else 8).  VEC: channel words per
+// thread; 2 (64-bit loads and stores, an even number of channel words, 3x3 windows on at most two planes)
+// halves the number of load instructions, which is what bounds this kernel.
+template <int NB, int VEC = 1>
 __global__ __launch_bounds__(256) void pool_planes_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
                                                           int B, int H, int W, int cw, int bits, int win, int stride,
                                                           int pad, int Ho, int Wo) {
   const long long rows_in = (long long)B * H * W, rows_out = (long long)B * Ho * Wo;
-  const long long total = rows_out * cw;
+  const int cwv = cw / VEC;  // threads per output pixel
+  const long long total = rows_out * cwv;
   const bool small = total < 0x7fffffffLL;  // 32-bit index arithmetic (64-bit divisions cost ~100 instructions)
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (long long)gridDim.x * blockDim.x) {
     int wi, ox, oy, b;
     long long row;
     if (small) {
-      const uint32_t iu = (uint32_t)i, r32 = iu / (uint32_t)cw;
-      wi = (int)(iu - r32 * (uint32_t)cw);
+      const uint32_t iu = (uint32_t)i, r32 = iu / (uint32_t)cwv;
+      wi = (int)(iu - r32 * (uint32_t)cwv) * VEC;
       const uint32_t t = r32 / (uint32_t)Wo;
       ox = (int)(r32 - t * (uint32_t)Wo);
       b = (int)(t / (uint32_t)Ho);
       oy = (int)(t - (uint32_t)b * (uint32_t)Ho);
       row = r32;
     } else {
-      wi = (int)(i % cw);
-      row = i / cw;
+      wi = (int)(i % cwv) * VEC;
+      row = i / cwv;
       ox = (int)(row % Wo);
       oy = (int)((row / Wo) % Ho);
       b = (int)(row / ((long long)Wo * Ho));
+    }
+    if constexpr (VEC == 2) {
+      // two channel words per thread: the same window logic on both halves of 64-bit loads
+      uint2 v[9][2];
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const int iy = oy * stride + t / 3 - pad, ix = ox * stride + t % 3 - pad;
+        const bool ok = iy >= 0 && iy < H && ix >= 0 && ix < W;
+        const long long rin = ((long long)b * H + iy) * W + ix;
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+          v[t][p] = (ok && p < bits) ? *reinterpret_cast<const uint2 *>(in + p * rows_in * cw + rin * cw + wi)
+                                     : make_uint2(0u, 0u);
+      }
+      uint32_t m0x = 0, m0y = 0, m1x = 0, m1y = 0;
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const uint32_t ltx = (v[t][1].x & ~m1x) | (~(v[t][1].x ^ m1x) & v[t][0].x & ~m0x);
+        const uint32_t lty = (v[t][1].y & ~m1y) | (~(v[t][1].y ^ m1y) & v[t][0].y & ~m0y);
+        m0x = (m0x & ~ltx) | (v[t][0].x & ltx);
+        m1x = (m1x & ~ltx) | (v[t][1].x & ltx);
+        m0y = (m0y & ~lty) | (v[t][0].y & lty);
+        m1y = (m1y & ~lty) | (v[t][1].y & lty);
+      }
+      *reinterpret_cast<uint2 *>(out + row * cw + wi) = make_uint2(m0x, m0y);
+      if (bits > 1) *reinterpret_cast<uint2 *>(out + rows_out * cw + row * cw + wi) = make_uint2(m1x, m1y);
+      continue;
     }
     uint32_t m[NB];
 #pragma unroll
@@ -1013,7 +1043,13 @@ hipError_t launch_pool_planes(const uint32_t *in, uint32_t *out, int B, int H, i
   const int Ho = (H + 2 * pad - win) / stride + 1, Wo = (W + 2 * pad - win) / stride + 1;
   long long blocks = ((long long)B * Ho * Wo * cw + 255) / 256;
   if (blocks > 262144) blocks = 262144;
-  if (bits <= 2)
+  // 64-bit accesses need 8-byte aligned rows: an even number of channel words and 8-byte aligned buffers
+  const bool vec2 = bits <= 2 && win == 3 && (cw & 1) == 0 &&
+                    ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 7) == 0;
+  if (vec2)
+    hipLaunchKernelGGL((pool_planes_kernel<2, 2>), dim3((unsigned)((blocks + 1) / 2)), dim3(256), 0, s, in, out, B, H, W, cw,
+                       bits, win, stride, pad, Ho, Wo);
+  else if (bits <= 2)
     hipLaunchKernelGGL(pool_planes_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, in, out, B, H, W, cw, bits, win,
                        stride, pad, Ho, Wo);
   else
